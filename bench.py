@@ -1,0 +1,260 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X attention hot path.  Prints ONE JSON line on stdout.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+A "step" is one pass of the selected workload over one batch of synthetic input that is
+already resident in HBM.  Workloads (shapes are the BASELINE.json configs):
+    decode    paged decode attention, batch 64, 16/8 heads, ctx U[100,2048]       (config 2)
+    scatter   store_kvcache, 4096 tokens into 512 blocks x 256 slots              (config 1)
+    prefill   causal varlen prefill, 16 sequences, half with cached prefix        (config 3)
+    sampler   temperature sampling over 256 x 151,936 logits
+The line carries `roofline` (algorithmic bytes or flops of the dominant kernel per launch,
+divided by its average duration measured with HIP events on the launch stream) and
+`cpu_baseline` (the CPU oracle timed on this box's host cores on a bounded sample).
+Only one GPU is used; --gpus above 1 is refused.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "nano-vllm_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16
+
+
+def _event_time_ms(fn_list, steps, warmup):
+    """Run fn_list[i % len] for warmup + steps iterations; HIP-event time of the timed part."""
+    import torch
+    n = len(fn_list)
+    for i in range(warmup):
+        fn_list[i % n]()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fn_list[(warmup + i) % n]()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop)
+
+
+def _median_cpu_seconds(fn, repeats=5, warm=1):
+    for _ in range(warm):
+        fn()
+    times = []
+    for _ in range(repeats):
+        t = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t)
+    return statistics.median(times)
+
+
+# ----------------------------------------------------------------------------- workloads
+def bench_decode(args, dev):
+    import torch
+    import nanovllm_amd as nva
+    from nanovllm_amd import synthetic
+    pools = 4                      # rotate 1 GiB pools so the 256 MB Infinity Cache cannot serve re-reads
+    cases, fns, alg = [], [], []
+    for p in range(pools):
+        g = torch.Generator(device=dev).manual_seed(100 + p)
+        kc = torch.randn((1024, 256, 8, 128), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        vc = torch.randn((1024, 256, 8, 128), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        c = synthetic.decode_case(seed=p, cache=(kc, vc))
+        q, cl, bt = c.q.to(dev), c.context_lens.to(dev), c.block_tables.to(dev)
+        out = torch.empty((64, 1, 16, 128), dtype=torch.bfloat16, device=dev)
+        cases.append(c)
+        alg.append(c.algorithmic_bytes)
+        fns.append(lambda q=q, kc=kc, vc=vc, cl=cl, bt=bt, s=c.scale, out=out:
+                   nva.paged_decode_attention(q, kc, vc, cl, bt, s, out=out))
+    ms = _event_time_ms(fns, args.steps, args.warmup)
+    per_step_ms = ms / args.steps
+    mean_alg = sum(alg[(args.warmup + i) % pools] for i in range(args.steps)) / args.steps
+    gbps = mean_alg / (per_step_ms * 1e-3) / 1e9
+    tokens = sum(int(c.context_lens.sum()) for c in cases) / pools
+    result = {
+        "metric": "paged decode attention, achieved HBM GB/s (config 2)",
+        "value": round(gbps, 1), "unit": "GB/s",
+        "ms_per_step": round(per_step_ms, 5),
+        "config": {"workload": "paged_decode_attn config2: batch 64, 16q/8kv heads, head_dim 128, block 256, "
+                               "ctx U[100,2048], 4 rotating 1 GiB KV pools",
+                   "batch": 64, "kv_tokens_per_step": tokens},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "decode_split_kernel<2> + decode_merge_kernel",
+                     "algorithmic_bytes_per_launch": int(mean_alg)},
+    }
+
+    def cpu():
+        import oracle
+        c = cases[0]
+        kc, vc = c.k_cache.cpu(), c.v_cache.cpu()
+        sec = _median_cpu_seconds(lambda: oracle.paged_decode_attention(
+            c.q, kc, vc, c.context_lens, c.block_tables, c.scale, "sdpa"), repeats=5)
+        return {"value": round(alg[0] / sec / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": "config 2 full batch (64 sequences), bf16 torch SDPA on gathered pages, "
+                                          "median of 5", "seconds": round(sec, 4)}
+    return result, cpu
+
+
+def bench_scatter(args, dev):
+    import torch
+    import nanovllm_amd as nva
+    from nanovllm_amd import synthetic
+    pools = 4
+    fns, alg, cases = [], [], []
+    for p in range(pools):
+        c = synthetic.scatter_case(seed=p)
+        k, v, kc, vc, sm = (t.to(dev) for t in (c.key, c.value, c.k_cache, c.v_cache, c.slot_mapping))
+        cases.append(c)
+        alg.append(c.algorithmic_bytes)
+        fns.append(lambda k=k, v=v, kc=kc, vc=vc, sm=sm: nva.store_kvcache(k, v, kc, vc, sm))
+    ms = _event_time_ms(fns, args.steps, args.warmup)
+    per_step_ms = ms / args.steps
+    gbps = alg[0] / (per_step_ms * 1e-3) / 1e9
+    result = {
+        "metric": "store_kvcache, achieved HBM GB/s (config 1)", "value": round(gbps, 1), "unit": "GB/s",
+        "ms_per_step": round(per_step_ms, 5),
+        "config": {"workload": "store_kvcache config1: 4096 tokens x 8 kv heads x 128, 512 blocks x 256 slots, "
+                               "5% skipped", "tokens": 4096},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "store_kvcache_kernel",
+                     "algorithmic_bytes_per_launch": int(alg[0])},
+    }
+
+    def cpu():
+        import oracle
+        c = cases[0]
+        sec = _median_cpu_seconds(lambda: oracle.store_kvcache(c.key, c.value, c.k_cache, c.v_cache, c.slot_mapping),
+                                  repeats=7)
+        return {"value": round(alg[0] / sec / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": "config 1 full size, torch index_copy_, median of 7",
+                "seconds": round(sec, 5)}
+    return result, cpu
+
+
+def bench_prefill(args, dev):
+    import torch
+    import nanovllm_amd as nva
+    from nanovllm_amd import synthetic
+    c = synthetic.prefill_case(seed=0)
+    q, k, v, kc, vc = (t.to(dev) for t in (c.q, c.k, c.v, c.k_cache, c.v_cache))
+    cq, ck, sm, bt = (t.to(dev) for t in (c.cu_seqlens_q, c.cu_seqlens_k, c.slot_mapping, c.block_tables))
+    nva.store_kvcache(k, v, kc, vc, sm)
+    fn = lambda: nva.varlen_prefill_attention(q, kc, vc, cq, ck, c.max_seqlen_q, c.max_seqlen_k, c.scale,
+                                              block_table=bt)
+    ms = _event_time_ms([fn], args.steps, args.warmup)
+    per_step_ms = ms / args.steps
+    flops = c.algorithmic_flops
+    tflops = flops / (per_step_ms * 1e-3) / 1e12
+    result = {
+        "metric": "causal varlen prefill attention with prefix cache, achieved TFLOP/s (config 3)",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_step": round(per_step_ms, 5),
+        "config": {"workload": "varlen_prefill_attn config3: 16 sequences, Lq U[100,1024], half with 1-3 cached "
+                               "256-token prefix blocks, 16q/8kv heads, head_dim 128", "total_q": int(c.q.shape[0])},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "prefill_attn_kernel<paged>", "algorithmic_flops_per_launch": int(flops)},
+    }
+
+    def cpu():
+        import oracle
+        ek, ev = c.k_cache.clone(), c.v_cache.clone()
+        oracle.store_kvcache(c.k, c.v, ek, ev, c.slot_mapping)
+        sec = _median_cpu_seconds(lambda: oracle.varlen_prefill_attention(
+            c.q, None, None, c.cu_seqlens_q, c.cu_seqlens_k, c.scale, ek, ev, c.block_tables, "sdpa"), repeats=3)
+        return {"value": round(flops / sec / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": "config 3 full batch, bf16 torch SDPA with explicit lower-right mask, "
+                                          "median of 3", "seconds": round(sec, 3)}
+    return result, cpu
+
+
+def bench_sampler(args, dev):
+    import torch
+    import nanovllm_amd as nva
+    batch, vocab = 256, 151936
+    g = torch.Generator(device=dev).manual_seed(5)
+    sets = []
+    for p in range(4):
+        logits = (torch.randn((batch, vocab), generator=g, device=dev) * 2).to(torch.bfloat16)
+        sets.append(logits)
+    temps = torch.full((batch,), 0.6, device=dev)
+    fns = [lambda l=l, i=i: nva.sample(l, temps, None, seed=1, offset=i) for i, l in enumerate(sets)]
+    ms = _event_time_ms(fns, args.steps, args.warmup)
+    per_step_ms = ms / args.steps
+    alg = batch * vocab * 2
+    gbps = alg / (per_step_ms * 1e-3) / 1e9
+    result = {
+        "metric": "sampler (in-kernel noise), achieved HBM GB/s", "value": round(gbps, 1), "unit": "GB/s",
+        "ms_per_step": round(per_step_ms, 5),
+        "config": {"workload": "sampler: 256 rows x 151,936 bf16 logits, T=0.6, Philox noise in-kernel",
+                   "batch": batch},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "sampler_partials_kernel + sampler_argmax_kernel + sampler_pick_kernel",
+                     "algorithmic_bytes_per_launch": alg},
+    }
+
+    def cpu():
+        import oracle
+        l = sets[0][:64].cpu()
+        t = temps[:64].cpu()
+        noise = torch.empty(64, vocab).exponential_(1.0)
+        sec = _median_cpu_seconds(lambda: oracle.sample(l, t, noise), repeats=5)
+        return {"value": round(64 * vocab * 2 / sec / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": "64 of the 256 rows, eager torch sampler with pre-drawn noise, "
+                                          "median of 5", "seconds": round(sec, 4)}
+    return result, cpu
+
+
+WORKLOADS = {"decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
+DEFAULT_STEPS = {"decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="decode")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the hot path needs no collectives); "
+                 "run with --gpus 1")
+    if args.steps is None:
+        args.steps = DEFAULT_STEPS[args.workload]
+    if args.warmup is None:
+        args.warmup = max(3, args.steps // 10)
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible (the hot path has no CPU fallback)")
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    from nanovllm_amd import _lib
+    _lib.load()
+
+    result, cpu_fn = WORKLOADS[args.workload](args, dev)
+    line = {
+        "metric": result["metric"], "value": result["value"], "unit": result["unit"],
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": result["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic", "config": result["config"], "roofline": result["roofline"],
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_fn()
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

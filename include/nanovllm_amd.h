@@ -1,0 +1,148 @@
+/*
+ * nanovllm_amd -- C ABI of the MI355X (gfx950) attention hot path for nano-vllm.
+ *
+ * Every entry point borrows raw device pointers for the duration of one asynchronous
+ * launch on the HIP stream it is given.  The library never allocates or frees device
+ * memory, never synchronises and never reads device data on the host, so all calls are
+ * legal under stream capture.  Scratch memory is supplied by the caller (query its size
+ * with the *_workspace_bytes functions).  Arguments are validated on the host before any
+ * launch; a non-zero return means nothing was enqueued.
+ *
+ * Dtypes / geometry: bf16 tensors, int32 index tensors, head_dim 128, KV block size 256,
+ * num_heads / num_kv_heads in {1, 2, 4, 8}.  Anything else is rejected with
+ * NVA_ERR_UNSUPPORTED_GEOMETRY rather than served by a slow path.
+ *
+ * File:line citations name the reference (nano-vllm) interface each entry point replaces.
+ */
+#ifndef NANOVLLM_AMD_H
+#define NANOVLLM_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum nva_status {
+    NVA_OK = 0,
+    NVA_ERR_NULL_POINTER = 1,         /* a required pointer is NULL                         */
+    NVA_ERR_BAD_SHAPE = 2,            /* negative / inconsistent counts                     */
+    NVA_ERR_UNSUPPORTED_GEOMETRY = 3, /* head_dim, block_size or GQA group not built        */
+    NVA_ERR_BAD_STRIDE = 4,           /* row stride smaller than a row, or not 16-byte      */
+    NVA_ERR_MISALIGNED = 5,           /* base pointer not 16-byte aligned                   */
+    NVA_ERR_WORKSPACE_TOO_SMALL = 6,  /* workspace_bytes below *_workspace_bytes()          */
+    NVA_ERR_LAUNCH_FAILED = 7,        /* hipGetLastError() after the launch was not success */
+    NVA_ERR_NO_DEVICE = 8             /* no HIP device visible                              */
+};
+
+/* Library version, (major << 16) | minor. */
+int nva_version(void);
+
+/* Static, human-readable name of a status code (never NULL). */
+const char *nva_status_string(int status);
+
+/* Number of visible HIP devices; NVA_ERR_NO_DEVICE (and *count = 0) when there is none. */
+int nva_device_count(int *count);
+
+/*
+ * KV-cache slot scatter.  Replaces store_kvcache / store_kvcache_kernel
+ * (nanovllm/layers/attention.py:10-40).
+ *
+ * key/value: bf16 [n_tokens, num_kv_heads, head_dim], innermost two dims dense, row
+ * strides in ELEMENTS (value is a strided view of the fused qkv buffer in the model).
+ * k_cache/v_cache: bf16, addressed flat as [num_slots, num_kv_heads*head_dim].
+ * slot_mapping: int32 [n_tokens]; row i goes to cache row slot_mapping[i]; -1 skips the
+ * row.  Slots outside [0, num_slots) are skipped as well instead of written out of
+ * bounds.  Duplicate slots are safe; which row wins is unspecified (as in the reference).
+ * The copy is bit-exact.  n_tokens == 0 is a no-op.
+ */
+int nva_store_kvcache(const void *key, int64_t key_row_stride,
+                      const void *value, int64_t value_row_stride,
+                      void *k_cache, void *v_cache,
+                      const int32_t *slot_mapping,
+                      int32_t n_tokens, int32_t num_kv_heads, int32_t head_dim,
+                      int64_t num_slots, void *stream);
+
+/*
+ * Paged single-query (decode) attention.  Replaces the flash_attn_with_kvcache call of
+ * Attention.forward (nanovllm/layers/attention.py:71-74).
+ *
+ * q: bf16 [batch, num_heads, head_dim], row stride q_row_stride elements, heads dense.
+ * k_cache/v_cache: bf16 [num_blocks, block_size, num_kv_heads, head_dim], dense.
+ * block_tables: int32 [batch, max_blocks] with row stride bt_row_stride; only entries
+ * j < ceil(context_lens[b] / block_size) are dereferenced (the rest may be -1 or stale);
+ * an entry outside [0, num_blocks) contributes nothing instead of faulting.
+ * context_lens: int32 [batch]; 0 yields an all-zero output row.
+ * out: bf16 [batch, num_heads, head_dim] dense (the reference's [B,1,Hq,Dh]).
+ * workspace: at least nva_paged_decode_workspace_bytes() bytes, 16-byte aligned; holds
+ * split-K partials, contents need no initialisation.
+ * Launch geometry depends only on (batch, max_blocks, heads), never on device data.
+ */
+size_t nva_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads, int32_t head_dim,
+                                        int32_t max_blocks);
+
+int nva_paged_decode_attn(const void *q, int64_t q_row_stride,
+                          const void *k_cache, const void *v_cache,
+                          const int32_t *block_tables, int32_t bt_row_stride, int32_t max_blocks,
+                          const int32_t *context_lens,
+                          void *out, void *workspace, size_t workspace_bytes,
+                          int32_t batch, int32_t num_heads, int32_t num_kv_heads,
+                          int32_t head_dim, int32_t block_size, int32_t num_blocks,
+                          float scale, void *stream);
+
+/*
+ * Causal variable-length prefill attention, optionally reading K/V through the paged
+ * cache.  Replaces the flash_attn_varlen_func call of Attention.forward
+ * (nanovllm/layers/attention.py:64-70).
+ *
+ * q: bf16 [total_q, num_heads, head_dim], row stride q_row_stride elements.
+ * block_tables == NULL: k/v are packed bf16 [total_k, num_kv_heads, head_dim] with their
+ *   own row strides, sequence b owning rows cu_seqlens_k[b]..cu_seqlens_k[b+1].
+ * block_tables != NULL: k/v are ignored (may be NULL) and every sequence reads its
+ *   cu_seqlens_k[b+1]-cu_seqlens_k[b] logical positions from k_cache/v_cache through
+ *   block_tables[b] (int32 [batch, max_blocks], row stride bt_row_stride, -1 padded).
+ * The causal mask is aligned to the END of the keys: query i of a sequence sees keys
+ * j <= i + (Lk - Lq).  Empty query spans are no-ops.
+ * out: bf16 [total_q, num_heads, head_dim] dense.  max_seqlen_q bounds the launch grid.
+ */
+int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride,
+                            const void *k, int64_t k_row_stride,
+                            const void *v, int64_t v_row_stride,
+                            const void *k_cache, const void *v_cache,
+                            const int32_t *block_tables, int32_t bt_row_stride, int32_t max_blocks,
+                            const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k,
+                            int32_t batch, int32_t max_seqlen_q, int32_t max_seqlen_k,
+                            void *out,
+                            int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
+                            int32_t block_size, int32_t num_blocks,
+                            float scale, void *stream);
+
+/*
+ * Temperature / exponential-race sampler.  Replaces Sampler.forward
+ * (nanovllm/layers/sampler.py:10-15):
+ *     token[b] = argmax_i softmax(float(logits[b]) / T[b])[i] / max(E[b,i], 1e-10)
+ * with the first index winning ties.
+ *
+ * logits: bf16 [batch, vocab], row stride logits_row_stride elements.
+ * temperatures: fp32 [batch].  T == 0 selects greedy argmax(logits) for that row (an
+ * extension; the reference forbids T <= 1e-10, nanovllm/sampling_params.py:11).
+ * noise: fp32 [batch, vocab] Exp(1) draws (row stride noise_row_stride), or NULL to draw
+ * them inside the kernel from Philox4x32-10 keyed by (seed, offset, row, column).
+ * out_tokens: int64 [batch].
+ * workspace: at least nva_sample_workspace_bytes() bytes, 16-byte aligned.
+ */
+size_t nva_sample_workspace_bytes(int32_t batch, int32_t vocab);
+
+int nva_sample(const void *logits, int64_t logits_row_stride,
+               const float *temperatures,
+               const float *noise, int64_t noise_row_stride,
+               uint64_t seed, uint64_t offset,
+               int64_t *out_tokens,
+               void *workspace, size_t workspace_bytes,
+               int32_t batch, int32_t vocab, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NANOVLLM_AMD_H */

@@ -1,0 +1,275 @@
+// Causal variable-length prefill attention for gfx950 (MFMA bf16, fp32 accumulate).
+//
+// Replaces flash_attn_varlen_func as called by nanovllm/layers/attention.py:64-70, including
+// the prefix-cache case where K/V of every sequence are read through the block table.
+//
+// One workgroup of 4 wavefronts per (128-query tile, query head, sequence); wavefront w owns
+// 32 query rows.  Keys are walked in tiles of 64; a K tile and a V tile ([64][128] bf16,
+// rows padded to 272 B) are staged in LDS.  Everything is computed transposed so that a
+// query is a LANE (lane % 32) and keys / output dims live in that lane's registers:
+//     S^T = K * Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q^T (registers)
+//     O^T = V^T * P^T    A = V^T gathered from LDS, B = P^T straight from the S^T accumulators
+// The softmax state (running max, running sum) is therefore per lane, reductions over keys
+// are in-register, and the only cross-lane step is one exchange between lanes l and l^32,
+// which hold the two key halves of the same query.  The S^T accumulator layout (register i
+// of lane l = key 8*(i/4) + 4*(l/32) + i%4) is also a legal k-ordering for the B operand of
+// the second product as long as V^T uses the same key order, so P never leaves registers.
+//
+// The causal mask is aligned to the end of the keys: query i sees keys j <= i + (Lk - Lq).
+// Work: 4 * 128 flop per (query, visible key, head).
+#include "nva_common.h"
+
+#include <math.h>
+
+namespace nva {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+constexpr int kPfThreads = 256;
+constexpr int kPfBM = 128;            // queries per workgroup
+constexpr int kPfBN = 64;             // keys per LDS tile
+constexpr int kPfLd = kHeadDim + 8;   // padded LDS row, elements (272 B)
+
+struct PrefillArgs {
+    const bf16_t *q; int64_t q_row_stride;
+    const bf16_t *k; int64_t k_row_stride;
+    const bf16_t *v; int64_t v_row_stride;
+    const bf16_t *k_cache; const bf16_t *v_cache;
+    const int32_t *block_tables; int32_t bt_row_stride;
+    const int32_t *cu_seqlens_q; const int32_t *cu_seqlens_k;
+    bf16_t *out;
+    int32_t num_heads, num_kv_heads, num_blocks;
+    float scale_log2e;
+};
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 &u) { return __builtin_bit_cast(bf16x8_t, u); }
+
+template <bool kPaged>
+__global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillArgs a) {
+    const int mt = blockIdx.x;
+    const int h = blockIdx.y;
+    const int b = blockIdx.z;
+    const int q0 = a.cu_seqlens_q[b], k0 = a.cu_seqlens_k[b];
+    const int lq = a.cu_seqlens_q[b + 1] - q0;
+    const int lk = a.cu_seqlens_k[b + 1] - k0;
+    const int row0 = mt * kPfBM;
+    if (row0 >= lq) return;                              // also covers empty query spans
+    const int off = lk - lq;                             // bottom-right causal alignment
+    const int hkv = h / (a.num_heads / a.num_kv_heads);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int qi = lane & 31, hh = lane >> 5;
+    const int qrow = row0 + wave * 32 + qi;              // query index inside the sequence
+    const bool q_valid = qrow < lq;
+    const int qrow_c = min(qrow, lq - 1);
+
+    // Q^T fragments: B operand, column = this lane's query, k = dims 16*s + 8*hh + [0,8)
+    bf16x8_t qfrag[8];
+    {
+        const bf16_t *qp = a.q + static_cast<int64_t>(q0 + qrow_c) * a.q_row_stride + h * kHeadDim + 8 * hh;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) qfrag[s] = as_bf16x8(*reinterpret_cast<const uint4 *>(qp + 16 * s));
+    }
+
+    f32x16_t oacc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+    float m_run = -INFINITY;      // shared by lanes l and l^32
+    float l_run = 0.f;            // partial over this lane's key half
+
+    __shared__ __attribute__((aligned(16))) bf16_t sK[kPfBN * kPfLd];
+    __shared__ __attribute__((aligned(16))) bf16_t sV[kPfBN * kPfLd];
+
+    const int q_hi = min(row0 + kPfBM, lq) - 1;          // last query row of the tile
+    const int kv_end = min(lk, q_hi + off + 1);          // keys [0, kv_end) are visible to the tile
+    const int ntiles = kv_end > 0 ? (kv_end + kPfBN - 1) / kPfBN : 0;
+    const int wave_qmin = row0 + wave * 32;
+
+    for (int kt = 0; kt < ntiles; ++kt) {
+        __syncthreads();                                 // everyone is done with the previous tile
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int c = tid + kPfThreads * r;          // 1024 16-byte chunks per tile
+            const int key = c >> 4, ch = c & 15;
+            const int kk = min(kt * kPfBN + key, lk - 1);     // rows past the end are masked below
+            uint4 kd, vd;
+            if (kPaged) {
+                const int32_t blk = a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + (kk >> 8)];
+                if (static_cast<uint32_t>(blk) < static_cast<uint32_t>(a.num_blocks)) {
+                    const int64_t e = ((static_cast<int64_t>(blk) * kBlockSize + (kk & 255)) * a.num_kv_heads + hkv) *
+                                          kHeadDim + ch * 8;
+                    kd = *reinterpret_cast<const uint4 *>(a.k_cache + e);
+                    vd = *reinterpret_cast<const uint4 *>(a.v_cache + e);
+                } else {
+                    kd = make_uint4(0, 0, 0, 0);
+                    vd = kd;
+                }
+            } else {
+                const int64_t tok = static_cast<int64_t>(k0 + kk);
+                kd = *reinterpret_cast<const uint4 *>(a.k + tok * a.k_row_stride + hkv * kHeadDim + ch * 8);
+                vd = *reinterpret_cast<const uint4 *>(a.v + tok * a.v_row_stride + hkv * kHeadDim + ch * 8);
+            }
+            *reinterpret_cast<uint4 *>(&sK[key * kPfLd + ch * 8]) = kd;
+            *reinterpret_cast<uint4 *>(&sV[key * kPfLd + ch * 8]) = vd;
+        }
+        __syncthreads();
+
+        // ---- S^T = K Q^T for two 32-key sub-tiles ----------------------------------------
+        f32x16_t sacc[2];
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sacc[t2][i] = 0.f;
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const uint4 kf = *reinterpret_cast<const uint4 *>(&sK[(t2 * 32 + qi) * kPfLd + 16 * s + 8 * hh]);
+                sacc[t2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf), qfrag[s], sacc[t2], 0, 0, 0);
+            }
+        }
+
+        // ---- scale, causal mask, running softmax ------------------------------------------
+        const int key_base = kt * kPfBN + 4 * hh;
+        const int limit = qrow + off;                    // last key this query may see
+        const bool need_mask = (kt * kPfBN + kPfBN - 1) > (wave_qmin + off);
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float x = sacc[t2][i] * a.scale_log2e;
+                if (need_mask) {
+                    const int key = key_base + t2 * 32 + 8 * (i >> 2) + (i & 3);
+                    if (key > limit) x = -INFINITY;
+                }
+                sacc[t2][i] = x;
+                mloc = fmaxf(mloc, x);
+            }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+        const float m_new = fmaxf(m_run, mloc);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;    // no key seen yet: p = 0
+        const float alpha = exp2f(m_run - m_safe);
+        m_run = m_new;
+        float psum = 0.f;
+        uint4 pfrag[2][2];                               // [sub-tile][k-step of 16 keys]
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            float p[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                p[i] = exp2f(sacc[t2][i] - m_safe);
+                psum += p[i];
+            }
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+                pfrag[t2][s2] = make_uint4(pack_bf16x2(p[8 * s2 + 0], p[8 * s2 + 1]),
+                                           pack_bf16x2(p[8 * s2 + 2], p[8 * s2 + 3]),
+                                           pack_bf16x2(p[8 * s2 + 4], p[8 * s2 + 5]),
+                                           pack_bf16x2(p[8 * s2 + 6], p[8 * s2 + 7]));
+        }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+
+        // ---- O^T += V^T P^T ----------------------------------------------------------------
+        // A operand: row = output dim (dt*32 + qi), k slot (hh, i) = key 16*s2 + 8*(i/4) + 4*hh + i%4
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+            const int dim = dt * 32 + qi;
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2) {
+                    const int kbase = t2 * 32 + 16 * s2 + 4 * hh;
+                    uint32_t w[4];
+#pragma unroll
+                    for (int pr = 0; pr < 4; ++pr) {
+                        const int ka = kbase + 8 * (pr >> 1) + 2 * (pr & 1);
+                        const uint32_t lo = sV[ka * kPfLd + dim];
+                        const uint32_t hi = sV[(ka + 1) * kPfLd + dim];
+                        w[pr] = lo | (hi << 16);
+                    }
+                    const uint4 vf = make_uint4(w[0], w[1], w[2], w[3]);
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf), as_bf16x8(pfrag[t2][s2]),
+                                                                       oacc[dt], 0, 0, 0);
+                }
+        }
+    }
+
+    // ---- normalise and store: register i of tile dt = dim dt*32 + 8*(i/4) + 4*hh + i%4 ----
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (q_valid) {
+        bf16_t *op = a.out + (static_cast<int64_t>(q0 + qrow) * a.num_heads + h) * kHeadDim + 4 * hh;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                uint2 w;
+                w.x = pack_bf16x2(oacc[dt][4 * g4 + 0] * inv, oacc[dt][4 * g4 + 1] * inv);
+                w.y = pack_bf16x2(oacc[dt][4 * g4 + 2] * inv, oacc[dt][4 * g4 + 3] * inv);
+                *reinterpret_cast<uint2 *>(op + dt * 32 + 8 * g4) = w;
+            }
+    }
+}
+
+}  // namespace nva
+
+extern "C" int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride, const void *k, int64_t k_row_stride,
+                                       const void *v, int64_t v_row_stride, const void *k_cache,
+                                       const void *v_cache, const int32_t *block_tables, int32_t bt_row_stride,
+                                       int32_t max_blocks, const int32_t *cu_seqlens_q,
+                                       const int32_t *cu_seqlens_k, int32_t batch, int32_t max_seqlen_q,
+                                       int32_t max_seqlen_k, void *out, int32_t num_heads, int32_t num_kv_heads,
+                                       int32_t head_dim, int32_t block_size, int32_t num_blocks, float scale,
+                                       void *stream) {
+    using namespace nva;
+    if (batch < 0 || max_seqlen_q < 0 || max_seqlen_k < 0 || num_heads <= 0 || num_kv_heads <= 0)
+        return NVA_ERR_BAD_SHAPE;
+    if (head_dim != kHeadDim) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+    if (num_heads % num_kv_heads != 0) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+    if (batch == 0 || max_seqlen_q == 0) return NVA_OK;
+    if (batch > 65535 || num_heads > 65535) return NVA_ERR_BAD_SHAPE;
+    if (!q || !cu_seqlens_q || !cu_seqlens_k || !out) return NVA_ERR_NULL_POINTER;
+    const bool paged = block_tables != nullptr;
+    const int64_t dkv = static_cast<int64_t>(num_kv_heads) * head_dim;
+    if (paged) {
+        if (block_size != kBlockSize) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+        if (!k_cache || !v_cache) return NVA_ERR_NULL_POINTER;
+        if (max_blocks <= 0 || num_blocks <= 0) return NVA_ERR_BAD_SHAPE;
+        if (bt_row_stride < max_blocks) return NVA_ERR_BAD_STRIDE;
+        if (static_cast<int64_t>(max_blocks) * kBlockSize < max_seqlen_k) return NVA_ERR_BAD_SHAPE;
+        if (!aligned16(k_cache) || !aligned16(v_cache)) return NVA_ERR_MISALIGNED;
+    } else {
+        if (!k || !v) return NVA_ERR_NULL_POINTER;
+        if (k_row_stride < dkv || v_row_stride < dkv || k_row_stride % 8 != 0 || v_row_stride % 8 != 0)
+            return NVA_ERR_BAD_STRIDE;
+        if (!aligned16(k) || !aligned16(v)) return NVA_ERR_MISALIGNED;
+    }
+    if (q_row_stride < static_cast<int64_t>(num_heads) * head_dim || q_row_stride % 8 != 0)
+        return NVA_ERR_BAD_STRIDE;
+    if (!aligned16(q) || !aligned16(out)) return NVA_ERR_MISALIGNED;
+
+    PrefillArgs a;
+    a.q = static_cast<const bf16_t *>(q); a.q_row_stride = q_row_stride;
+    a.k = static_cast<const bf16_t *>(k); a.k_row_stride = k_row_stride;
+    a.v = static_cast<const bf16_t *>(v); a.v_row_stride = v_row_stride;
+    a.k_cache = static_cast<const bf16_t *>(k_cache); a.v_cache = static_cast<const bf16_t *>(v_cache);
+    a.block_tables = block_tables; a.bt_row_stride = bt_row_stride;
+    a.cu_seqlens_q = cu_seqlens_q; a.cu_seqlens_k = cu_seqlens_k;
+    a.out = static_cast<bf16_t *>(out);
+    a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.num_blocks = num_blocks;
+    a.scale_log2e = scale * 1.4426950408889634f;
+    const dim3 grid((max_seqlen_q + kPfBM - 1) / kPfBM, num_heads, batch);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (paged)
+        hipLaunchKernelGGL(prefill_attn_kernel<true>, grid, dim3(kPfThreads), 0, s, a);
+    else
+        hipLaunchKernelGGL(prefill_attn_kernel<false>, grid, dim3(kPfThreads), 0, s, a);
+    return launch_status();
+}

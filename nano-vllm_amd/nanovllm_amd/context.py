@@ -1,0 +1,50 @@
+"""Per-step side channel between the model runner and the attention layers.
+
+Same contract as nanovllm/utils/context.py:5-27: a module-global record that the runner
+replaces before each forward pass (``set_context``), the attention layers and the LM head
+read (``get_context``) and the runner clears afterwards (``reset_context``).  Field names,
+defaults and the positional order of ``set_context`` are the reference's
+(nanovllm/engine/model_runner.py:160 passes eight positionals).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+
+@dataclass
+class Context:
+    """Tensors describing the batch being run.  Index tensors are int32 on the device.
+
+    prefill: cu_seqlens_q/k ``[B+1]``, max_seqlen_q/k, slot_mapping ``[total_q]`` and, only
+             when some sequence reads cached prefix blocks, block_tables ``[B, max_blocks]``.
+    decode:  slot_mapping ``[B]``, context_lens ``[B]``, block_tables ``[B, max_blocks]``.
+    """
+    is_prefill: bool = False
+    cu_seqlens_q: Optional[torch.Tensor] = None
+    cu_seqlens_k: Optional[torch.Tensor] = None
+    max_seqlen_q: int = 0
+    max_seqlen_k: int = 0
+    slot_mapping: Optional[torch.Tensor] = None
+    context_lens: Optional[torch.Tensor] = None
+    block_tables: Optional[torch.Tensor] = None
+
+
+class _Holder:
+    current = Context()
+
+
+def get_context() -> Context:
+    return _Holder.current
+
+
+def set_context(is_prefill, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=0, max_seqlen_k=0,
+                slot_mapping=None, context_lens=None, block_tables=None) -> None:
+    _Holder.current = Context(is_prefill, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                              slot_mapping, context_lens, block_tables)
+
+
+def reset_context() -> None:
+    _Holder.current = Context()

@@ -1,0 +1,63 @@
+"""Token sampler backed by the fused gfx950 kernels.
+
+Drop-in for nanovllm/layers/sampler.py: ``Sampler()(logits, temperatures) -> int64 [B]``,
+an exact categorical draw from ``softmax(logits / T)`` via the exponential race
+``argmax(p / E)``, ``E ~ Exp(1)``.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import _lib
+
+
+def sample(logits: torch.Tensor, temperatures: torch.Tensor, noise: Optional[torch.Tensor] = None,
+           seed: int = 0, offset: int = 0) -> torch.Tensor:
+    """``argmax(softmax(logits.float() / T) / clamp_min(E, 1e-10))`` per row.
+
+    ``noise`` (fp32 ``[B, V]``) supplies ``E`` explicitly so a draw can be replayed; with
+    ``noise=None`` the kernel draws ``E`` itself from Philox keyed by ``(seed, offset)``.
+    Rows with temperature 0 return ``argmax(logits)``.
+    """
+    assert logits.dim() == 2 and logits.dtype == torch.bfloat16 and logits.stride(1) == 1
+    b, vocab = logits.shape
+    assert temperatures.dtype == torch.float32 and temperatures.numel() == b and temperatures.is_contiguous()
+    if not logits.is_cuda:
+        raise RuntimeError("nanovllm_amd ops run on the GPU only (there is no CPU fallback)")
+    out = torch.empty(b, dtype=torch.int64, device=logits.device)
+    if b == 0:
+        return out
+    if noise is not None:
+        assert noise.dtype == torch.float32 and noise.shape == logits.shape and noise.stride(1) == 1
+        assert noise.is_cuda
+    lib = _lib.load()
+    nbytes = lib.nva_sample_workspace_bytes(b, vocab)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=logits.device)
+    rc = lib.nva_sample(logits.data_ptr(), logits.stride(0), temperatures.data_ptr(),
+                        None if noise is None else noise.data_ptr(),
+                        0 if noise is None else noise.stride(0),
+                        int(seed) & 0xFFFFFFFFFFFFFFFF, int(offset) & 0xFFFFFFFFFFFFFFFF,
+                        out.data_ptr(), ws.data_ptr(), ws.numel(), b, vocab,
+                        torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "nva_sample")
+    return out
+
+
+class Sampler(nn.Module):
+    """``forward(logits, temperatures)`` as in nanovllm/layers/sampler.py:10-15.
+
+    Each call advances a Philox offset, so successive calls draw fresh noise while a run
+    with the same ``seed`` is reproducible.
+    """
+
+    def __init__(self, seed: int = 0):
+        super().__init__()
+        self.seed = seed
+        self.calls = 0
+
+    def forward(self, logits: torch.Tensor, temperatures: torch.Tensor) -> torch.Tensor:
+        self.calls += 1
+        return sample(logits, temperatures, None, self.seed, self.calls)

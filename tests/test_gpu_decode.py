@@ -1,0 +1,117 @@
+"""Paged decode attention on the GPU, through the C ABI, against the fp32 oracle."""
+import pytest
+import torch
+
+import oracle
+from nanovllm_amd import paged_decode_attention
+from nanovllm_amd import synthetic
+from helpers import assert_attn_close, bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu(case, dev, tables=None):
+    t = case.block_tables if tables is None else tables
+    out = paged_decode_attention(case.q.to(dev), case.k_cache.to(dev), case.v_cache.to(dev),
+                                 case.context_lens.to(dev), t.to(dev), case.scale)
+    torch.cuda.synchronize()
+    return out
+
+
+def _oracle(case):
+    return oracle.paged_decode_attention(case.q, case.k_cache, case.v_cache, case.context_lens,
+                                         case.block_tables, case.scale, "fp32")
+
+
+def test_decode_config2(dev):
+    """batch 64, 16 q / 8 kv heads, head_dim 128, ctx U[100,2048], 1024-block pool."""
+    case = synthetic.decode_case(seed=0)
+    out = _gpu(case, dev)
+    assert out.shape == (64, 1, 16, 128) and out.dtype == torch.bfloat16
+    assert_attn_close(out, _oracle(case), "config 2")
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (8, 8), (16, 2), (8, 1)])
+def test_decode_gqa_groups(dev, hq, hkv):
+    case = synthetic.decode_case(seed=hq * 10 + hkv, batch=9, num_heads=hq, num_kv_heads=hkv, num_blocks=64,
+                                 ctx_lo=1, ctx_hi=1200)
+    assert_attn_close(_gpu(case, dev), _oracle(case), f"gqa {hq}/{hkv}")
+
+
+def test_decode_edge_context_lengths(dev):
+    lens = [0, 1, 2, 63, 64, 65, 255, 256, 257, 511, 512, 513, 1024, 0, 3]
+    case = synthetic.decode_case(seed=7, num_blocks=64, context_lens=lens)
+    out = _gpu(case, dev)
+    want = _oracle(case)
+    assert_attn_close(out, want, "edge lens")
+    assert not out[0].any() and not out[13].any()              # context_len 0 -> zeros
+    # one key: the output is exactly that V row (bf16 round trip of fp32 is the identity)
+    blk = int(case.block_tables[1, 0])
+    assert torch.equal(bits(out[1, 0, 0]), bits(case.v_cache[blk, 0, 0]))
+    assert torch.equal(bits(out[1, 0, 1]), bits(case.v_cache[blk, 0, 0]))     # heads 0,1 -> kv head 0
+    assert torch.equal(bits(out[1, 0, 15]), bits(case.v_cache[blk, 0, 7]))
+
+
+def test_decode_ignores_stale_and_padded_table_entries(dev):
+    """Only entries j < ceil(ctx/256) may be dereferenced: the rest may be -1, stale ids of
+    other sequences, or out-of-range garbage (graph replays never clear the table)."""
+    case = synthetic.decode_case(seed=8, batch=12, num_blocks=64, ctx_lo=1, ctx_hi=1500)
+    base = _gpu(case, dev)
+    wide = torch.full((12, 16), -1, dtype=torch.int32)
+    wide[:, : case.block_tables.shape[1]] = case.block_tables
+    need = (case.context_lens + 255) // 256
+    g = torch.Generator().manual_seed(1)
+    for b in range(12):
+        n = int(need[b])
+        junk = torch.randint(0, 64, (16 - n,), generator=g, dtype=torch.int32)
+        junk[::3] = 1 << 30
+        junk[1::3] = -5
+        wide[b, n:] = junk
+    out = _gpu(case, dev, wide)
+    assert torch.equal(bits(out), bits(base))
+    assert_attn_close(out, _oracle(case), "stale tables")
+
+
+def test_decode_invariants(dev):
+    case = synthetic.decode_case(seed=9, batch=8, num_blocks=48, ctx_lo=200, ctx_hi=1100)
+    out = _gpu(case, dev)
+    # V == 1 -> out == 1
+    ones = synthetic.DecodeCase(case.q, case.k_cache, torch.ones_like(case.v_cache), case.context_lens,
+                                case.block_tables, case.scale)
+    o1 = _gpu(ones, dev).float().cpu()
+    assert (o1 - 1).abs().max() < 1e-2
+    # renaming physical blocks changes nothing, bit for bit
+    perm = torch.randperm(48, generator=torch.Generator().manual_seed(2))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(48)
+    t2 = torch.where(case.block_tables >= 0, inv[case.block_tables.clamp_min(0).long()].to(torch.int32),
+                     case.block_tables)
+    moved = synthetic.DecodeCase(case.q, case.k_cache[perm], case.v_cache[perm], case.context_lens, t2, case.scale)
+    assert torch.equal(bits(_gpu(moved, dev)), bits(out))
+    # garbage beyond context_len inside the last block is never used
+    kc, vc = case.k_cache.clone(), case.v_cache.clone()
+    for b in range(8):
+        n = int(case.context_lens[b])
+        last = int(case.block_tables[b, (n - 1) // 256])
+        kc[last, n % 256 if n % 256 else 256:] = float("nan")
+        vc[last, n % 256 if n % 256 else 256:] = float("inf")
+    dirty = synthetic.DecodeCase(case.q, kc, vc, case.context_lens, case.block_tables, case.scale)
+    assert torch.equal(bits(_gpu(dirty, dev)), bits(out))
+
+
+def test_decode_long_context_many_splits(dev):
+    """Qwen3-8B geometry (32/8 heads), 65-wide tables, contexts up to 16384."""
+    lens = [16384, 4096, 9001, 12345]
+    case = synthetic.decode_case(seed=11, num_heads=32, num_kv_heads=8, num_blocks=180, context_lens=lens)
+    assert_attn_close(_gpu(case, dev), _oracle(case), "long ctx")
+
+
+def test_decode_q_as_4d_and_strided(dev):
+    case = synthetic.decode_case(seed=12, batch=5, num_blocks=32, ctx_lo=10, ctx_hi=700)
+    qkv = torch.zeros(5, 16 * 128 + 2 * 8 * 128, dtype=torch.bfloat16)
+    qkv[:, : 16 * 128] = case.q.reshape(5, -1)
+    qd = qkv.to(dev)[:, : 16 * 128].view(5, 16, 128)            # row stride 4096
+    out = paged_decode_attention(qd.unsqueeze(1), case.k_cache.to(dev), case.v_cache.to(dev),
+                                 case.context_lens.to(dev), case.block_tables.to(dev), case.scale)
+    torch.cuda.synchronize()
+    assert_attn_close(out, _oracle(case), "strided q")

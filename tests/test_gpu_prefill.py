@@ -1,0 +1,120 @@
+"""Causal varlen prefill attention on the GPU, through the C ABI, against the fp32 oracle."""
+import pytest
+import torch
+
+import oracle
+from nanovllm_amd import varlen_prefill_attention, store_kvcache
+from nanovllm_amd import synthetic
+from helpers import assert_attn_close, bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _paged(case, dev):
+    """scatter the new keys, then attend through the block table -- what Attention.forward does"""
+    kc, vc = case.k_cache.to(dev), case.v_cache.to(dev)
+    store_kvcache(case.k.to(dev), case.v.to(dev), kc, vc, case.slot_mapping.to(dev))
+    out = varlen_prefill_attention(case.q.to(dev), kc, vc, case.cu_seqlens_q.to(dev), case.cu_seqlens_k.to(dev),
+                                   case.max_seqlen_q, case.max_seqlen_k, case.scale,
+                                   block_table=case.block_tables.to(dev))
+    torch.cuda.synchronize()
+    ek, ev = case.k_cache.clone(), case.v_cache.clone()
+    oracle.store_kvcache(case.k, case.v, ek, ev, case.slot_mapping)
+    want = oracle.varlen_prefill_attention(case.q, None, None, case.cu_seqlens_q, case.cu_seqlens_k, case.scale,
+                                           ek, ev, case.block_tables, "fp32")
+    return out, want
+
+
+def _packed(case, dev, strided_v=False):
+    k, v = case.k.to(dev), case.v.to(dev)
+    if strided_v:
+        n, hkv, dh = case.v.shape
+        wide = torch.zeros(n, 4 * hkv * dh, dtype=torch.bfloat16, device=dev)
+        wide[:, 3 * hkv * dh:] = v.reshape(n, -1)
+        v = wide[:, 3 * hkv * dh:].view(n, hkv, dh)
+    out = varlen_prefill_attention(case.q.to(dev), k, v, case.cu_seqlens_q.to(dev), case.cu_seqlens_k.to(dev),
+                                   case.max_seqlen_q, case.max_seqlen_k, case.scale)
+    torch.cuda.synchronize()
+    want = oracle.varlen_prefill_attention(case.q, case.k, case.v, case.cu_seqlens_q, case.cu_seqlens_k,
+                                           case.scale, precision="fp32")
+    return out, want
+
+
+def test_prefill_config3_prefix_cache(dev):
+    """16 sequences, Lq U[100,1024], half with 1-3 cached 256-token prefix blocks."""
+    case = synthetic.prefill_case(seed=0)
+    assert case.block_tables is not None and sum(1 for p in case.prefix_lens if p) == 8
+    out, want = _paged(case, dev)
+    assert out.shape == case.q.shape
+    assert_attn_close(out, want, "config 3")
+
+
+@pytest.mark.parametrize("strided_v", [False, True])
+def test_prefill_no_prefix_packed(dev, strided_v):
+    case = synthetic.prefill_case(seed=1, batch=6, prefix_fraction=0.0, q_lo=1, q_hi=700)
+    assert case.block_tables is None
+    out, want = _packed(case, dev, strided_v)
+    assert_attn_close(out, want, "packed")
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (8, 8), (4, 1)])
+def test_prefill_gqa_groups(dev, hq, hkv):
+    case = synthetic.prefill_case(seed=hq, batch=4, num_heads=hq, num_kv_heads=hkv, q_lo=5, q_hi=400, num_blocks=24)
+    out, want = _paged(case, dev)
+    assert_attn_close(out, want, f"gqa {hq}/{hkv}")
+
+
+def test_prefill_ragged_lengths_and_tile_edges(dev):
+    q_lens = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300]
+    prefix = [0, 1, 0, 2, 0, 0, 1, 0, 3, 0, 1, 0, 0, 2, 1]
+    case = synthetic.prefill_case(seed=2, q_lens=q_lens, prefix_blocks=prefix, num_blocks=48)
+    out, want = _paged(case, dev)
+    assert_attn_close(out, want, "ragged paged")
+    case2 = synthetic.prefill_case(seed=3, q_lens=q_lens, prefix_blocks=[0] * len(q_lens), num_blocks=48)
+    out2, want2 = _packed(case2, dev)
+    assert_attn_close(out2, want2, "ragged packed")
+    # first token of every sequence sees one key only: output is exactly that V row
+    for s in range(len(q_lens)):
+        a = int(case2.cu_seqlens_q[s])
+        assert torch.equal(bits(out2[a, 0]), bits(case2.v[a, 0]))
+        assert torch.equal(bits(out2[a, 15]), bits(case2.v[a, 7]))
+
+
+def test_prefill_lq1_with_prefix_equals_decode_semantics(dev):
+    case = synthetic.prefill_case(seed=4, q_lens=[1, 1, 1], prefix_blocks=[1, 3, 2], num_blocks=16)
+    out, want = _paged(case, dev)
+    assert_attn_close(out, want, "lq=1")
+
+
+def test_prefill_empty_query_span_is_a_noop(dev):
+    """A prompt fully covered by cached blocks has seqlen_q == 0 (two equal cu_seqlens_q)."""
+    case = synthetic.prefill_case(seed=5, q_lens=[40, 70], prefix_blocks=[1, 0], num_blocks=16)
+    cu_q = torch.tensor([0, 40, 40, 110], dtype=torch.int32)
+    cu_k = torch.tensor([0, 296, 296 + 512, 296 + 512 + 70], dtype=torch.int32)
+    tables = torch.full((3, 2), -1, dtype=torch.int32)
+    tables[0, :2] = case.block_tables[0, :2]
+    tables[1, :2] = torch.tensor([14, 15], dtype=torch.int32)         # fully cached sequence
+    tables[2, :1] = case.block_tables[1, :1]
+    kc, vc = case.k_cache.to(dev), case.v_cache.to(dev)
+    store_kvcache(case.k.to(dev), case.v.to(dev), kc, vc, case.slot_mapping.to(dev))
+    out = varlen_prefill_attention(case.q.to(dev), kc, vc, cu_q.to(dev), cu_k.to(dev), 70, 512, case.scale,
+                                   block_table=tables.to(dev))
+    torch.cuda.synchronize()
+    ek, ev = case.k_cache.clone(), case.v_cache.clone()
+    oracle.store_kvcache(case.k, case.v, ek, ev, case.slot_mapping)
+    want = oracle.varlen_prefill_attention(case.q, None, None, cu_q, cu_k, case.scale, ek, ev, tables, "fp32")
+    assert_attn_close(out, want, "empty span")
+
+
+def test_prefill_sequences_do_not_leak(dev):
+    case = synthetic.prefill_case(seed=6, batch=3, prefix_fraction=0.0, q_lo=50, q_hi=200)
+    out, _ = _packed(case, dev)
+    k2 = case.k.clone()
+    a, b = int(case.cu_seqlens_q[1]), int(case.cu_seqlens_q[2])
+    k2[a:b] = 2.0
+    case2 = synthetic.PrefillCase(case.q, k2, case.v, case.k_cache, case.v_cache, case.cu_seqlens_q,
+                                  case.cu_seqlens_k, case.max_seqlen_q, case.max_seqlen_k, case.slot_mapping,
+                                  None, case.scale)
+    out2, _ = _packed(case2, dev)
+    assert torch.equal(bits(out[:a]), bits(out2[:a])) and torch.equal(bits(out[b:]), bits(out2[b:]))
+    assert not torch.equal(bits(out[a:b]), bits(out2[a:b]))
