@@ -53,15 +53,17 @@ def test_scatter_empty_and_all_skipped(dev):
 
 
 def test_scatter_duplicate_slots_are_safe(dev):
-    """Graph capture runs with slot_mapping == 0 for every row: no fault, slot 0 holds one
-    of the rows, everything else untouched."""
+    """Graph capture runs with slot_mapping == 0 for every row: no fault, slot 0 holds
+    pieces of the competing rows, everything else untouched."""
     case = synthetic.scatter_case(seed=4, n_tokens=128, num_blocks=2, skip_fraction=0.0)
     kc, vc = case.k_cache.to(dev), case.v_cache.to(dev)
     store_kvcache(case.key.to(dev), case.value.to(dev), kc, vc, torch.zeros(128, dtype=torch.int32, device=dev))
     torch.cuda.synchronize()
     assert not kc.view(-1, 1024)[1:].any() and not vc.view(-1, 1024)[1:].any()
-    row = bits(kc.view(-1, 1024)[0])
-    assert any(torch.equal(row, bits(case.key[i].reshape(-1))) for i in range(128))
+    # rows race chunk by chunk: every 16-byte chunk of slot 0 is the same chunk of SOME token
+    got = bits(kc.view(-1, 1024)[0]).view(128, 8)
+    src = bits(case.key.reshape(128, 1024)).view(128, 128, 8)          # [token, chunk, 8]
+    assert bool((got.unsqueeze(0) == src).all(-1).any(0).all())
 
 
 def test_scatter_out_of_range_slots_are_skipped(dev):
