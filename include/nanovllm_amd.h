@@ -76,8 +76,10 @@ int nva_store_kvcache(const void *key, int64_t key_row_stride,
  * context_lens: int32 [batch]; 0 yields an all-zero output row.
  * out: bf16 [batch, num_heads, head_dim] dense (the reference's [B,1,Hq,Dh]).
  * workspace: at least nva_paged_decode_workspace_bytes() bytes, 16-byte aligned; holds
- * split-K partials, contents need no initialisation.
- * Launch geometry depends only on (batch, max_blocks, heads), never on device data.
+ * split partials, contents need no initialisation.  Calls that overlap in time need
+ * separate workspaces; calls ordered on one stream (every layer of a model) can share one.
+ * Launch geometry depends only on (batch, heads), never on device data, so a call can be
+ * captured in a HIP graph and replayed with new contents.
  */
 size_t nva_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads, int32_t head_dim,
                                         int32_t max_blocks);

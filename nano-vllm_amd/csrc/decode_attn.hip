@@ -1,239 +1,421 @@
-// Paged single-query (decode) attention for gfx950: split-K over 256-token KV blocks.
+// Paged single-query (decode) attention for gfx950: persistent, evenly split stream of KV.
 //
 // Replaces flash_attn_with_kvcache as called by nanovllm/layers/attention.py:71-74.
 //
-// Stage 1 (decode_split_kernel): one workgroup of 4 wavefronts per
-// (KV block j of the sequence, kv head g, sequence b).  Wavefront w owns tokens
-// [64w, 64w+64) of the block.  A K (or V) head row is 128 bf16 = 256 B = 16 lanes x 16 B, so a
-// wavefront reads 4 token rows per dwordx4 load instruction; it issues all 16 K loads and
-// all 16 V loads of its 64 tokens up front (32 KB in flight per wavefront) and only then
-// starts the arithmetic, which keeps the memory pipe full without any software pipeline.
-// The G = num_heads/num_kv_heads query heads that share kv head g are processed together
-// from the same registers (K and V are read once per kv head, not once per query head).
-// Scores are reduced over the 16 lanes of a row with DPP adds; the softmax is the usual
-// running-max form in base 2 (scale * log2(e) folded into q).  The four wavefronts merge
-// through LDS and write one unnormalised partial (max, sum, o[128]) per query head.
-// Stage 2 (decode_merge_kernel): one workgroup per (query head, sequence) merges the
-// ceil(ctx/256) partials and writes bf16.
+// Work decomposition.  The unit of work is a "stage": 32 consecutive tokens of one kv head of
+// one sequence (8 KB of K + 8 KB of V; a stage never straddles a 256-token KV block).  All
+// stages of the batch form one list ordered by (sequence, kv head, position) -- its length N
+// follows from context_lens alone, which every workgroup prefix-sums in LDS.  The launch is
+// a fixed set of W = 2048 wavefront "workers" (512 workgroups x 4) and worker w takes the
+// contiguous slice [w*N/W, (w+1)*N/W) (one stage each when N < W): every worker streams the same number of bytes
+// whatever the mix of context lengths, nothing is launched for empty table entries, and
+// the 8 XCDs (which receive workgroups round-robin) stay balanced.  The grid depends on no
+// device data, so the launch can be captured in a HIP graph and replayed with new contents.
+//
+// Per worker, a two-deep software pipeline over its stages:
+//   * HBM -> VGPR: a K (or V) head row is 128 bf16 = 256 B = 16 lanes x 16 B, so one dwordx4
+//     load instruction covers 4 full token rows; a stage is 8 K + 8 V loads per lane, and
+//     the loads of stage x+1 are issued before the arithmetic of stage x, so every resident
+//     wavefront keeps 16 KB in flight all the time (128 KB per CU at 8 wavefronts).
+//   * VGPR -> LDS: rows go to a wavefront-private 16 KB region with an XOR swizzle of the
+//     16-byte chunk index, so the matrix-core operand reads below are free of bank
+//     conflicts although the row pitch is exactly 256 B.  No workgroup barrier is needed.
+//   * S^T = K Q^T: v_mfma_f32_16x16x32_bf16, A = 16 token rows from LDS, B = Q^T in
+//     registers; the G = num_heads/num_kv_heads query heads sharing the kv head are the
+//     first G of the 16 columns (the rest are zero), so K is read once per kv head.
+//   * softmax in base 2 on the accumulator layout (lane = head, registers = tokens): running
+//     max / sum per lane, one exchange across the four 16-lane groups per stage.
+//   * O^T += V^T P^T: A = V^T through ds_read_b64_tr_b16 (LDS transpose read: 4 tokens x 16
+//     dims -> lane = dim, registers = tokens), B = P^T straight from the S^T registers.
+// When a worker leaves a (sequence, kv head) pair it either writes the final bf16 rows (it
+// saw all of the pair's stages) or an unnormalised partial (max, sum, o[128]) per query
+// head.  A second, small kernel (decode_merge_kernel) merges the partials of the pairs that
+// were split over several workers; the kernel boundary is the only synchronisation (device
+// wide fences inside the streaming kernel cost far more than the boundary: they flush the
+// L2 of the XCD).
 //
 // HBM traffic per sequence and layer: ctx * num_kv_heads * 128 * 2 B for K plus the same for
-// V (4096 B per token at 8 kv heads); partials add (128+2)*4 B per (block, query head), 1.6 %.
-//
-// Launch geometry is a function of (batch, max_blocks, heads) only; context_lens and the
-// block table are read on the device, so the launch can be captured in a HIP graph and
-// replayed with new contents.  Workgroups whose block lies beyond context_lens[b] exit at
-// once; only block_tables[b][j] with j*256 < context_lens[b] is dereferenced.
+// V (4096 B per token at 8 kv heads).  Partials: at most (W + batch*num_kv_heads) * G rows of 520 B.
 #include "nva_common.h"
 
 #include <math.h>
 
 namespace nva {
 
-constexpr int kSplitThreads = 256;
-constexpr int kTokPerWave = 64;
-constexpr int kIters = kTokPerWave / 4;   // 4 token rows per load instruction
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));   // plain vectors: stay in registers
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kDecThreads = 256;
+constexpr int kDecWaves = kDecThreads / kWave;
+constexpr int kDecGrid = 512;                       // workgroups; 2 per CU on a 256-CU part
+constexpr int kDecWorkers = kDecGrid * kDecWaves;   // wavefront workers
+constexpr int kDecMaxBatch = 1024;                  // sequences per launch (prefix sums live in LDS)
+constexpr int kStageTok = 32;                       // tokens per stage
+constexpr int kStagesPerBlock = kBlockSize / kStageTok;
+constexpr int kStageLoads = kStageTok / 4;          // dwordx4 loads per lane per stage and tensor
+constexpr int kWaveLdsChunks = 2 * kStageTok * 16;  // K then V, in 16-byte chunks
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(const u32x4_t &u) { return __builtin_bit_cast(bf16x8_t, u); }
+
+// the worker that owns stage x when n stages are split over nw <= n workers as [w*n/nw, (w+1)*n/nw)
+__device__ __forceinline__ int worker_of(int64_t x, int64_t n, int64_t nw) {
+    return static_cast<int>(((x + 1) * nw - 1) / n);
+}
+
+struct DecodeArgs {
+    const bf16_t *q; int64_t q_row_stride;
+    const bf16_t *k_cache; const bf16_t *v_cache;
+    const int32_t *block_tables; int32_t bt_row_stride;
+    const int32_t *context_lens;
+    bf16_t *out;
+    int32_t *pref_out;       // [batch + 1] stage-count prefix sums, written for the merge kernel
+    float *part_ml;          // [rows][2]
+    float *part_o;           // [rows][128]
+    int32_t batch, max_blocks, num_heads, num_kv_heads, num_blocks;
+    float scale_log2e;
+};
 
 template <int G>
-__global__ __launch_bounds__(kSplitThreads) void decode_split_kernel(
-    const bf16_t *__restrict__ q, int64_t q_row_stride,
-    const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
-    const int32_t *__restrict__ block_tables, int32_t bt_row_stride,
-    const int32_t *__restrict__ context_lens,
-    float *__restrict__ part_o, float *__restrict__ part_ml,
-    int32_t max_blocks, int32_t num_heads, int32_t num_kv_heads, int32_t num_blocks,
-    float scale_log2e) {
-    const int j = blockIdx.x;
-    const int g = blockIdx.y;
-    const int b = blockIdx.z;
-    const int ctx = context_lens[b];
-    const int blk_tok0 = j * kBlockSize;
-    if (blk_tok0 >= ctx) return;                       // uniform for the whole workgroup
-    const int32_t blk = block_tables[static_cast<int64_t>(b) * bt_row_stride + j];
-    const bool blk_ok = static_cast<uint32_t>(blk) < static_cast<uint32_t>(num_blocks);
-    const int n_blk = min(kBlockSize, ctx - blk_tok0); // valid tokens in this block, >= 1
-
+__global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const DecodeArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int tg = lane >> 4;                           // token row within a load instruction
-    const int dl = lane & 15;                           // 16-byte chunk of the head row
-    const int w0 = wave * kTokPerWave;
+    const int grp = lane >> 4;     // 16-lane group: token row of a load, k-slot group of an MFMA
+    const int r16 = lane & 15;     // chunk of a load; token / head / dim index of an MFMA operand
+    const int hkv = a.num_kv_heads;
 
-    float m_w[G], l_w[G], o[G][8];
+    // ---- stage-count prefix sums over the batch (every workgroup computes its own copy) -------
+    __shared__ int32_t sh_pref[kDecMaxBatch + 1];   // sh_pref[b] = stages of all (sequence < b, head)
+    __shared__ __attribute__((aligned(16))) u32x4_t lds[kDecWaves * kWaveLdsChunks];
+    if (wave == 0) {
+        constexpr int kPer = kDecMaxBatch / kWave;  // 16 sequences per lane
+        int cnt[kPer];
+        int local = 0;
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-        m_w[h] = -INFINITY;
-        l_w[h] = 0.f;
-#pragma unroll
-        for (int d = 0; d < 8; ++d) o[h][d] = 0.f;
-    }
-
-    if (blk_ok && w0 < n_blk) {
-        const int last = n_blk - 1;
-        const int64_t row = static_cast<int64_t>(num_kv_heads) * kHeadDim;   // elements per token
-        const int64_t base = static_cast<int64_t>(blk) * kBlockSize * row + g * kHeadDim + dl * 8;
-        const bf16_t *kb = k_cache + base;
-        const bf16_t *vb = v_cache + base;
-        uint4 kr[kIters], vr[kIters];
-#pragma unroll
-        for (int i = 0; i < kIters; ++i) {
-            const int t = min(w0 + i * 4 + tg, last);   // clamp: stay on rows that were written
-            kr[i] = *reinterpret_cast<const uint4 *>(kb + t * row);
-        }
-#pragma unroll
-        for (int i = 0; i < kIters; ++i) {
-            const int t = min(w0 + i * 4 + tg, last);
-            vr[i] = *reinterpret_cast<const uint4 *>(vb + t * row);
-        }
-
-        float qf[G][8];
-#pragma unroll
-        for (int h = 0; h < G; ++h) {
-            const bf16_t *qp = q + static_cast<int64_t>(b) * q_row_stride + (g * G + h) * kHeadDim + dl * 8;
-            const uint4 qr = *reinterpret_cast<const uint4 *>(qp);
-            unpack8(qr, qf[h]);
-#pragma unroll
-            for (int d = 0; d < 8; ++d) qf[h][d] *= scale_log2e;
-        }
-
-        float s[kIters][G];
-#pragma unroll
-        for (int i = 0; i < kIters; ++i) {
-            float kf[8];
-            unpack8(kr[i], kf);
-            const bool valid = (w0 + i * 4 + tg) <= last;
-#pragma unroll
-            for (int h = 0; h < G; ++h) {
-                float acc = 0.f;
-#pragma unroll
-                for (int d = 0; d < 8; ++d) acc = fmaf(qf[h][d], kf[d], acc);
-                acc = row16_sum(acc);
-                s[i][h] = valid ? acc : -INFINITY;
+        for (int i = 0; i < kPer; ++i) {
+            const int b = lane * kPer + i;
+            int c = 0;
+            if (b < a.batch) {
+                const int ctx = a.context_lens[b];
+                const int st = ctx > 0 ? (ctx + kStageTok - 1) / kStageTok : 0;
+                // a context that does not fit the table is clipped to it instead of read out of bounds
+                c = min(st, a.max_blocks * kStagesPerBlock) * hkv;
             }
+            cnt[i] = c;
+            local += c;
         }
+        int incl = local;                            // inclusive scan over the 64 lanes
 #pragma unroll
-        for (int h = 0; h < G; ++h) {
-            float mx = s[0][h];
-#pragma unroll
-            for (int i = 1; i < kIters; ++i) mx = fmaxf(mx, s[i][h]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));   // finite: token w0 of this wave is valid
-            float sum = 0.f;
-#pragma unroll
-            for (int i = 0; i < kIters; ++i) {
-                s[i][h] = exp2f(s[i][h] - mx);
-                sum += s[i][h];
-            }
-            sum += __shfl_xor(sum, 16, 64);
-            sum += __shfl_xor(sum, 32, 64);
-            m_w[h] = mx;
-            l_w[h] = sum;
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += up;
         }
+        int run = incl - local;
+        if (lane == 0) sh_pref[0] = 0;
 #pragma unroll
-        for (int i = 0; i < kIters; ++i) {
-            float vf[8];
-            unpack8(vr[i], vf);
-#pragma unroll
-            for (int h = 0; h < G; ++h)
-#pragma unroll
-                for (int d = 0; d < 8; ++d) o[h][d] = fmaf(s[i][h], vf[d], o[h][d]);
-        }
-#pragma unroll
-        for (int h = 0; h < G; ++h)
-#pragma unroll
-            for (int d = 0; d < 8; ++d) {
-                o[h][d] += __shfl_xor(o[h][d], 16, 64);
-                o[h][d] += __shfl_xor(o[h][d], 32, 64);
-            }
-    }
-
-    // ---- merge the four wavefronts through LDS ------------------------------------------
-    __shared__ float sh_m[4][G];
-    __shared__ float sh_l[4][G];
-    __shared__ float sh_o[4][G][kHeadDim];
-    if (tg == 0) {
-#pragma unroll
-        for (int h = 0; h < G; ++h)
-#pragma unroll
-            for (int d = 0; d < 8; ++d) sh_o[wave][h][dl * 8 + d] = o[h][d];
-    }
-    if (lane == 0) {
-#pragma unroll
-        for (int h = 0; h < G; ++h) {
-            sh_m[wave][h] = m_w[h];
-            sh_l[wave][h] = l_w[h];
+        for (int i = 0; i < kPer; ++i) {
+            run += cnt[i];
+            sh_pref[lane * kPer + i + 1] = run;      // entries past the batch repeat the total
         }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < G * kHeadDim; idx += kSplitThreads) {
-        const int h = idx / kHeadDim;
-        const int d = idx % kHeadDim;
-        float m = sh_m[0][h];
+    const int64_t n_total = sh_pref[a.batch];
+    if (blockIdx.x == 0)
+        for (int i = threadIdx.x; i <= a.batch; i += kDecThreads) a.pref_out[i] = sh_pref[i];
+
+    // ---- sequences with no keys produce zero rows -----------------------------------------------
+    for (int b = blockIdx.x; b < a.batch; b += gridDim.x) {
+        if (sh_pref[b + 1] == sh_pref[b]) {
+            const int chunks = a.num_heads * kHeadDim / 8;
+            u32x4_t *dst = reinterpret_cast<u32x4_t *>(a.out + static_cast<int64_t>(b) * a.num_heads * kHeadDim);
+            for (int c = threadIdx.x; c < chunks; c += kDecThreads) dst[c] = u32x4_t{0u, 0u, 0u, 0u};
+        }
+    }
+
+    // With fewer stages than workers only the first n_total workers get (one) stage each, so that
+    // the workers of a pair are always consecutive.
+    const int w = blockIdx.x * kDecWaves + wave;
+    const int64_t n_workers = n_total < kDecWorkers ? n_total : kDecWorkers;
+    if (w >= n_workers) return;                      // wave-uniform; no barrier follows
+    const int64_t lo = static_cast<int64_t>(w) * n_total / n_workers;
+    const int64_t hi = static_cast<int64_t>(w + 1) * n_total / n_workers;   // > lo
+
+    u32x4_t *sK = lds + wave * kWaveLdsChunks;
+    u32x4_t *sV = sK + kStageTok * 16;
+    const int64_t row = static_cast<int64_t>(hkv) * kHeadDim;       // elements per token row
+
+    // ---- locate the first stage: largest b with sh_pref[b] <= lo --------------------------------
+    int b;
+    {
+        int l = 0, r = a.batch;                      // invariant: sh_pref[l] <= lo < sh_pref[r]
+        while (r - l > 1) {
+            const int mid = (l + r) >> 1;
+            if (sh_pref[mid] <= lo) l = mid; else r = mid;
+        }
+        b = l;
+    }
+    int nst = (sh_pref[b + 1] - sh_pref[b]) / hkv;   // stages per head of sequence b (> 0)
+    int g = static_cast<int>(lo - sh_pref[b]) / nst;
+    int s = static_cast<int>(lo - sh_pref[b]) % nst;
+
+    // HBM -> registers for stage (bb, gg, ss) of a sequence with nn stages per head.  Token rows
+    // are clamped to the last valid row of the stage, so only rows that were written are touched.
+    auto load_stage = [&](int bb, int gg, int ss, int nn, u32x4_t (&kr)[kStageLoads], u32x4_t (&vr)[kStageLoads],
+                          u32x4_t (&qr)[4], int &last) __attribute__((always_inline)) {
+        const int ctx = min(a.context_lens[bb], nn * kStageTok);
+        last = min(kStageTok, ctx - ss * kStageTok) - 1;                       // in [0, 31]
+        int32_t blk = a.block_tables[static_cast<int64_t>(bb) * a.bt_row_stride + ss / kStagesPerBlock];
+        if (static_cast<uint32_t>(blk) >= static_cast<uint32_t>(a.num_blocks)) {
+            blk = 0;                                  // bad table entry: contributes nothing
+            last = -1;
+        }
+        const int tok0 = (ss % kStagesPerBlock) * kStageTok;
+        const int64_t base = (static_cast<int64_t>(blk) * kBlockSize + tok0) * row + gg * kHeadDim + r16 * 8;
+        const bf16_t *kb = a.k_cache + base;
+        const bf16_t *vb = a.v_cache + base;
+        const int lastc = max(last, 0);
 #pragma unroll
-        for (int w = 1; w < 4; ++w) m = fmaxf(m, sh_m[w][h]);
-        float l = 0.f, acc = 0.f;
-        if (m > -INFINITY) {
+        for (int i = 0; i < kStageLoads; ++i) {
+            const int t = min(i * 4 + grp, lastc);
+            kr[i] = *reinterpret_cast<const u32x4_t *>(kb + t * row);
+            vr[i] = *reinterpret_cast<const u32x4_t *>(vb + t * row);
+        }
+        // Q^T fragments (B operand): column = head r16 (zero beyond G), k-slots = dims 32i + 8grp + [0,8)
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const float f = exp2f(sh_m[w][h] - m);   // exp2(-inf) = 0 for idle wavefronts
-                l = fmaf(f, sh_l[w][h], l);
-                acc = fmaf(f, sh_o[w][h][d], acc);
+        for (int i = 0; i < 4; ++i) {
+            u32x4_t u = {0u, 0u, 0u, 0u};
+            if (r16 < G)
+                u = *reinterpret_cast<const u32x4_t *>(a.q + static_cast<int64_t>(bb) * a.q_row_stride +
+                                                       (gg * G + r16) * kHeadDim + 32 * i + 8 * grp);
+            qr[i] = u;
+        }
+    };
+
+    f32x4_t oacc[8];               // O^T: lane = head r16, tile dt register i = dim 16dt + 4grp + i
+    float m_run, l_run;
+    auto reset_state = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) oacc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        m_run = -INFINITY;
+        l_run = 0.f;
+    };
+    reset_state();
+
+    u32x4_t kr[kStageLoads], vr[kStageLoads], qr[4];
+    int last;
+    load_stage(b, g, s, nst, kr, vr, qr, last);
+
+    for (int64_t x = lo; x < hi; ++x) {
+        // ---- registers -> LDS (swizzled) ------------------------------------------------------
+#pragma unroll
+        for (int i = 0; i < kStageLoads; ++i) {
+            const int t = i * 4 + grp;
+            sK[t * 16 + (r16 ^ (t & 15))] = kr[i];
+            sV[t * 16 + (r16 ^ (2 * (t & 7)))] = vr[i];
+        }
+        bf16x8_t qf[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) qf[i] = as_bf16x8(qr[i]);
+        const int cur_last = last;
+        const int cur_b = b, cur_g = g, cur_nst = nst;
+
+        // ---- coordinates of the next stage; its loads fly during this stage's arithmetic ------
+        const bool more = x + 1 < hi;
+        bool pair_ends = true;
+        if (more) {
+            if (s + 1 < nst) {
+                ++s;
+                pair_ends = false;
+            } else {
+                s = 0;
+                if (g + 1 < hkv) {
+                    ++g;
+                } else {
+                    g = 0;
+                    do { ++b; } while (sh_pref[b + 1] == sh_pref[b]);   // skip sequences without keys
+                    nst = (sh_pref[b + 1] - sh_pref[b]) / hkv;
+                }
+            }
+            load_stage(b, g, s, nst, kr, vr, qr, last);
+        }
+        __builtin_amdgcn_wave_barrier();
+
+        // ---- S^T = K Q^T: two tiles of 16 tokens ------------------------------------------------
+        f32x4_t sc[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            sc[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const u32x4_t ka = sK[(16 * tt + r16) * 16 + ((4 * i + grp) ^ r16)];
+                sc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ka), qf[i], sc[tt], 0, 0, 0);
             }
         }
-        const int64_t slot = (static_cast<int64_t>(b) * max_blocks + j) * num_heads + g * G + h;
-        part_o[slot * kHeadDim + d] = acc;
-        if (d == 0) {
-            part_ml[slot * 2 + 0] = m;
-            part_ml[slot * 2 + 1] = l;
+        // register i of tile tt = token 16tt + 4grp + i of the stage
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float v = (16 * tt + 4 * grp + i <= cur_last) ? sc[tt][i] * a.scale_log2e : -INFINITY;
+                sc[tt][i] = v;
+                mloc = fmaxf(mloc, v);
+            }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+        const float m_new = fmaxf(m_run, mloc);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;     // nothing visible yet: p = 0, alpha = 0
+        const float alpha = exp2f(m_run - m_use);
+        m_run = m_new;
+        float p[8];
+        float psum = 0.f;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p[4 * tt + i] = exp2f(sc[tt][i] - m_use);
+                psum += p[4 * tt + i];
+            }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) oacc[dt] *= alpha;
+        // P^T as B operand: k-slot i = token 4grp + i, k-slot 4+i = token 16 + 4grp + i
+        const u32x4_t pu = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]),
+                            pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7])};
+        const bf16x8_t pf = as_bf16x8(pu);
+
+        // ---- O^T += V^T P^T -----------------------------------------------------------------------
+        // transpose read: the 16 lanes of a group fetch [4 tokens][16 dims]; lane r16 supplies the
+        // address of token r16/4, dims 4*(r16%4)..+3 and receives dim r16 of the four tokens
+        {
+            const int t_lo = 4 * grp + (r16 >> 2);
+            const int t_hi = t_lo + 16;
+            const int sub = (r16 >> 1) & 1;            // which 16-byte chunk of the 32-byte dim span
+            const char *vbase = reinterpret_cast<const char *>(sV) + (r16 & 1) * 8;
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) {
+                const int c = 2 * dt + sub;
+                const s16x4_t vlo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4_ptr)(vbase + t_lo * 256 + ((c ^ (2 * (t_lo & 7))) * 16)));
+                const s16x4_t vhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4_ptr)(vbase + t_hi * 256 + ((c ^ (2 * (t_hi & 7))) * 16)));
+                const s16x8_t both = __builtin_shufflevector(vlo, vhi, 0, 1, 2, 3, 4, 5, 6, 7);
+                oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), pf,
+                                                                   oacc[dt], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();               // this stage's LDS reads precede the next stage's writes
+
+        // ---- leaving the (sequence, kv head) pair: final rows, or a partial for the merge --------
+        if (pair_ends) {
+            float l_tot = l_run + __shfl_xor(l_run, 16, 64);
+            l_tot += __shfl_xor(l_tot, 32, 64);
+            const int64_t pair_lo = sh_pref[cur_b] + static_cast<int64_t>(cur_g) * cur_nst;   // first stage of the pair
+            const int64_t pair_hi = pair_lo + cur_nst;
+            if (lo <= pair_lo && pair_hi <= hi) {      // this worker saw the whole pair
+                if (r16 < G) {
+                    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+                    bf16_t *op = a.out + (static_cast<int64_t>(cur_b) * a.num_heads + cur_g * G + r16) * kHeadDim + 4 * grp;
+#pragma unroll
+                    for (int dt = 0; dt < 8; ++dt) {
+                        const u32x2_t o2 = {pack_bf16x2(oacc[dt][0] * inv, oacc[dt][1] * inv),
+                                            pack_bf16x2(oacc[dt][2] * inv, oacc[dt][3] * inv)};
+                        *reinterpret_cast<u32x2_t *>(op + 16 * dt) = o2;
+                    }
+                }
+            } else {
+                const int pair = cur_b * hkv + cur_g;
+                const int64_t slot = static_cast<int64_t>(w) + pair;   // unique per (worker, pair) along the stage list
+                if (r16 < G) {
+                    float *po = a.part_o + (slot * G + r16) * kHeadDim + 4 * grp;
+#pragma unroll
+                    for (int dt = 0; dt < 8; ++dt) *reinterpret_cast<f32x4_t *>(po + 16 * dt) = oacc[dt];
+                    if (grp == 0) {
+                        a.part_ml[(slot * G + r16) * 2 + 0] = m_run;
+                        a.part_ml[(slot * G + r16) * 2 + 1] = l_tot;
+                    }
+                }
+            }
+            reset_state();
         }
     }
 }
 
-// One workgroup of 128 lanes (lane = output dim) per (query head, sequence).
-__global__ __launch_bounds__(kHeadDim) void decode_merge_kernel(
-    const float *__restrict__ part_o, const float *__restrict__ part_ml,
-    const int32_t *__restrict__ context_lens, bf16_t *__restrict__ out,
-    int32_t max_blocks, int32_t num_heads) {
-    const int h = blockIdx.x;
-    const int b = blockIdx.y;
-    const int d = threadIdx.x;
-    const int ctx = context_lens[b];
-    const int nsplit = min(max_blocks, (ctx + kBlockSize - 1) / kBlockSize);
-    const int64_t first = (static_cast<int64_t>(b) * max_blocks) * num_heads + h;
-    float m = -INFINITY;
-    for (int j = 0; j < nsplit; ++j) m = fmaxf(m, part_ml[(first + static_cast<int64_t>(j) * num_heads) * 2]);
-    float acc = 0.f, l = 0.f;
-    if (m > -INFINITY) {
-        for (int j = 0; j < nsplit; ++j) {
-            const int64_t slot = first + static_cast<int64_t>(j) * num_heads;
-            const float f = exp2f(part_ml[slot * 2] - m);
-            l = fmaf(f, part_ml[slot * 2 + 1], l);
-            acc = fmaf(f, part_o[slot * kHeadDim + d], acc);
+// Merges the partials of every (sequence, kv head) pair that was split over several workers.
+// One workgroup of G wavefronts per pair: wavefront h merges query head g*G + h, lane = 2 dims.
+// It recomputes which workers met the pair from the stage-count prefix sums the streaming
+// kernel left in the workspace; pairs seen by a single worker were already written.
+template <int G>
+__global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArgs a) {
+    const int pair = blockIdx.x;
+    const int b = pair / a.num_kv_heads;
+    const int g = pair % a.num_kv_heads;
+    const int h = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int64_t n_total = a.pref_out[a.batch];
+    const int pb = a.pref_out[b];
+    const int nst = (a.pref_out[b + 1] - pb) / a.num_kv_heads;
+    if (nst == 0) return;                              // no keys: the zero rows are already there
+    const int64_t n_workers = n_total < kDecWorkers ? n_total : kDecWorkers;
+    const int64_t pair_lo = pb + static_cast<int64_t>(g) * nst;
+    const int w_first = worker_of(pair_lo, n_total, n_workers);
+    const int n_parts = worker_of(pair_lo + nst - 1, n_total, n_workers) - w_first + 1;
+    if (n_parts == 1) return;                          // one worker saw the whole pair and wrote it
+    const int64_t row0 = (static_cast<int64_t>(w_first) + pair) * G + h;   // rows of consecutive workers are G apart
+    float mx = -INFINITY;
+    for (int pi = lane; pi < n_parts; pi += kWave) mx = fmaxf(mx, a.part_ml[(row0 + static_cast<int64_t>(pi) * G) * 2]);
+    mx = wave_max(mx);
+    float acc0 = 0.f, acc1 = 0.f, lsum = 0.f;
+    if (mx > -INFINITY) {
+        for (int pi = 0; pi < n_parts; ++pi) {
+            const int64_t at = row0 + static_cast<int64_t>(pi) * G;
+            const float f = exp2f(a.part_ml[at * 2] - mx);
+            lsum = fmaf(f, a.part_ml[at * 2 + 1], lsum);
+            const float2 o2 = *reinterpret_cast<const float2 *>(a.part_o + at * kHeadDim + 2 * lane);
+            acc0 = fmaf(f, o2.x, acc0);
+            acc1 = fmaf(f, o2.y, acc1);
         }
     }
-    const float r = l > 0.f ? acc / l : 0.f;             // no visible key -> zeros
-    out[(static_cast<int64_t>(b) * num_heads + h) * kHeadDim + d] = f32_to_bf16(r);
+    const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+    *reinterpret_cast<uint32_t *>(a.out + (static_cast<int64_t>(b) * a.num_heads + g * G + h) * kHeadDim + 2 * lane) =
+        pack_bf16x2(acc0 * inv, acc1 * inv);
 }
 
 template <int G>
-static void launch_split(const void *q, int64_t q_row_stride, const void *k_cache, const void *v_cache,
-                         const int32_t *block_tables, int32_t bt_row_stride, const int32_t *context_lens,
-                         float *part_o, float *part_ml, int32_t max_blocks, int32_t batch,
-                         int32_t num_heads, int32_t num_kv_heads, int32_t num_blocks, float scale_log2e,
-                         hipStream_t stream) {
-    hipLaunchKernelGGL(decode_split_kernel<G>, dim3(max_blocks, num_kv_heads, batch), dim3(kSplitThreads),
-                       0, stream, static_cast<const bf16_t *>(q), q_row_stride,
-                       static_cast<const bf16_t *>(k_cache), static_cast<const bf16_t *>(v_cache),
-                       block_tables, bt_row_stride, context_lens, part_o, part_ml, max_blocks, num_heads,
-                       num_kv_heads, num_blocks, scale_log2e);
+static int launch_decode(const DecodeArgs &a, hipStream_t stream) {
+    hipLaunchKernelGGL(decode_stream_kernel<G>, dim3(kDecGrid), dim3(kDecThreads), 0, stream, a);
+    if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
+    hipLaunchKernelGGL(decode_merge_kernel<G>, dim3(a.batch * a.num_kv_heads), dim3(G * kWave), 0, stream, a);
+    return launch_status();
+}
+
+static inline size_t align_up(size_t v, size_t to) { return (v + to - 1) / to * to; }
+
+struct DecodeWorkspace {
+    size_t pref_bytes, rows, total;
+};
+static DecodeWorkspace decode_workspace(int32_t batch, int32_t num_heads, int32_t head_dim) {
+    DecodeWorkspace ws;
+    const size_t per_launch = static_cast<size_t>(batch < kDecMaxBatch ? batch : kDecMaxBatch);
+    ws.pref_bytes = align_up((per_launch + 1) * sizeof(int32_t), 256);
+    // partial rows: one per query head of every (worker, pair) met along the stage list;
+    // row index = (worker + pair) * G + head < W * G + batch * num_heads, and G <= 8
+    ws.rows = static_cast<size_t>(kDecWorkers) * (num_heads < 8 ? num_heads : 8) + per_launch * num_heads;
+    ws.total = ws.pref_bytes + ws.rows * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
+    return ws;
 }
 
 }  // namespace nva
 
 extern "C" size_t nva_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads, int32_t head_dim,
                                                    int32_t max_blocks) {
-    if (batch <= 0 || num_heads <= 0 || head_dim <= 0 || max_blocks <= 0) return 0;
-    const size_t slots = static_cast<size_t>(batch) * max_blocks * num_heads;
-    return slots * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
+    (void)max_blocks;
+    if (batch <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
+    return nva::decode_workspace(batch, num_heads, head_dim).total;
 }
 
 extern "C" int nva_paged_decode_attn(const void *q, int64_t q_row_stride, const void *k_cache,
@@ -251,39 +433,47 @@ extern "C" int nva_paged_decode_attn(const void *q, int64_t q_row_stride, const 
     const int group = num_heads / num_kv_heads;
     if (group != 1 && group != 2 && group != 4 && group != 8) return NVA_ERR_UNSUPPORTED_GEOMETRY;
     if (batch == 0) return NVA_OK;
-    if (batch > 65535 || num_kv_heads > 65535) return NVA_ERR_BAD_SHAPE;      // grid y/z limits
-    if (!q || !k_cache || !v_cache || !context_lens || !out) return NVA_ERR_NULL_POINTER;
-    if (max_blocks > 0 && (!block_tables || !workspace)) return NVA_ERR_NULL_POINTER;
+    if (static_cast<int64_t>(max_blocks) * kStagesPerBlock * num_kv_heads * kDecMaxBatch > 0x7fffffffLL)
+        return NVA_ERR_BAD_SHAPE;                                             // stage counts are int32
+    if (!q || !k_cache || !v_cache || !context_lens || !out || !workspace) return NVA_ERR_NULL_POINTER;
+    if (max_blocks > 0 && !block_tables) return NVA_ERR_NULL_POINTER;
     if (q_row_stride < static_cast<int64_t>(num_heads) * head_dim || q_row_stride % 8 != 0)
         return NVA_ERR_BAD_STRIDE;
     if (bt_row_stride < max_blocks) return NVA_ERR_BAD_STRIDE;
-    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(workspace))
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(workspace) || !aligned16(out))
         return NVA_ERR_MISALIGNED;
-    if (workspace_bytes < nva_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks))
-        return NVA_ERR_WORKSPACE_TOO_SMALL;
+    const DecodeWorkspace ws = decode_workspace(batch, num_heads, head_dim);
+    if (workspace_bytes < ws.total) return NVA_ERR_WORKSPACE_TOO_SMALL;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const size_t slots = static_cast<size_t>(batch) * max_blocks * num_heads;
-    float *part_o = static_cast<float *>(workspace);
-    float *part_ml = part_o + slots * kHeadDim;
-    const float scale_log2e = scale * 1.4426950408889634f;
-    if (max_blocks > 0) {
+    DecodeArgs a;
+    a.k_cache = static_cast<const bf16_t *>(k_cache);
+    a.v_cache = static_cast<const bf16_t *>(v_cache);
+    a.bt_row_stride = bt_row_stride;
+    a.q_row_stride = q_row_stride;
+    a.pref_out = static_cast<int32_t *>(workspace);
+    a.part_ml = reinterpret_cast<float *>(static_cast<char *>(workspace) + ws.pref_bytes);
+    a.part_o = a.part_ml + ws.rows * 2;
+    a.max_blocks = max_blocks;
+    a.num_heads = num_heads;
+    a.num_kv_heads = num_kv_heads;
+    a.num_blocks = num_blocks;
+    a.scale_log2e = scale * 1.4426950408889634f;
+    // launches of at most kDecMaxBatch sequences each, back to back on the stream
+    for (int32_t b0 = 0; b0 < batch; b0 += kDecMaxBatch) {
+        a.batch = batch - b0 < kDecMaxBatch ? batch - b0 : kDecMaxBatch;
+        a.q = static_cast<const bf16_t *>(q) + static_cast<int64_t>(b0) * q_row_stride;
+        a.block_tables = block_tables + static_cast<int64_t>(b0) * bt_row_stride;
+        a.context_lens = context_lens + b0;
+        a.out = static_cast<bf16_t *>(out) + static_cast<int64_t>(b0) * num_heads * head_dim;
+        int rc;
         switch (group) {
-#define NVA_CASE(G)                                                                                      \
-    case G:                                                                                              \
-        launch_split<G>(q, q_row_stride, k_cache, v_cache, block_tables, bt_row_stride, context_lens,    \
-                        part_o, part_ml, max_blocks, batch, num_heads, num_kv_heads, num_blocks,         \
-                        scale_log2e, s);                                                                 \
-        break;
-            NVA_CASE(1)
-            NVA_CASE(2)
-            NVA_CASE(4)
-            NVA_CASE(8)
-#undef NVA_CASE
+            case 1: rc = launch_decode<1>(a, s); break;
+            case 2: rc = launch_decode<2>(a, s); break;
+            case 4: rc = launch_decode<4>(a, s); break;
+            default: rc = launch_decode<8>(a, s); break;
         }
-        if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
+        if (rc != NVA_OK) return rc;
     }
-    hipLaunchKernelGGL(decode_merge_kernel, dim3(num_heads, batch), dim3(kHeadDim), 0, s, part_o, part_ml,
-                       context_lens, static_cast<bf16_t *>(out), max_blocks, num_heads);
-    return launch_status();
+    return NVA_OK;
 }

@@ -39,7 +39,7 @@ struct PrefillArgs {
     const int32_t *block_tables; int32_t bt_row_stride;
     const int32_t *cu_seqlens_q; const int32_t *cu_seqlens_k;
     bf16_t *out;
-    int32_t num_heads, num_kv_heads, num_blocks;
+    int32_t num_heads, num_kv_heads, num_blocks, num_q_tiles;
     float scale_log2e;
 };
 
@@ -47,9 +47,12 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 &u) { return __builtin
 
 template <bool kPaged>
 __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillArgs a) {
-    const int mt = blockIdx.x;
-    const int h = blockIdx.y;
-    const int b = blockIdx.z;
+    // Workgroups go to the 8 XCDs round-robin by linear id, so the head is the fastest index
+    // (every XCD gets the same mix of tiles however ragged the sequences are) and the query
+    // tiles run from the last one (most keys, longest) to the first.
+    const int h = blockIdx.x % a.num_heads;
+    const int mt = a.num_q_tiles - 1 - (blockIdx.x / a.num_heads) % a.num_q_tiles;
+    const int b = blockIdx.x / (a.num_heads * a.num_q_tiles);
     const int q0 = a.cu_seqlens_q[b], k0 = a.cu_seqlens_k[b];
     const int lq = a.cu_seqlens_q[b + 1] - q0;
     const int lk = a.cu_seqlens_k[b + 1] - k0;
@@ -265,7 +268,9 @@ extern "C" int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride, cons
     a.out = static_cast<bf16_t *>(out);
     a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.num_blocks = num_blocks;
     a.scale_log2e = scale * 1.4426950408889634f;
-    const dim3 grid((max_seqlen_q + kPfBM - 1) / kPfBM, num_heads, batch);
+    a.num_q_tiles = (max_seqlen_q + kPfBM - 1) / kPfBM;
+    if (static_cast<int64_t>(a.num_q_tiles) * num_heads * batch > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;
+    const dim3 grid(static_cast<uint32_t>(a.num_q_tiles) * num_heads * batch);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (paged)
         hipLaunchKernelGGL(prefill_attn_kernel<true>, grid, dim3(kPfThreads), 0, s, a);

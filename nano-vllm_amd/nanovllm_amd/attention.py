@@ -62,13 +62,18 @@ def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor,
 _workspaces: dict = {}
 
 
-def _decode_workspace(device, nbytes: int, under_capture: bool) -> torch.Tensor:
-    """Split-K scratch.  Outside graph capture one growing buffer per device is reused;
-    under capture a fresh tensor is taken from the graph's private pool."""
-    if under_capture:
-        return torch.empty(nbytes, dtype=torch.uint8, device=device)
+def _decode_workspace(device, nbytes: int) -> torch.Tensor:
+    """Scratch for the decode kernel's split partials.
+
+    One buffer per device, shared by every layer (calls are ordered on one stream).  It
+    only grows outside graph capture: a captured graph
+    must be preceded by an eager warm-up call of the same shape, which is what the runner
+    does before capturing each batch size (nanovllm/engine/model_runner.py:232-234).
+    """
     ws = _workspaces.get(device)
     if ws is None or ws.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("decode workspace must be allocated by an eager warm-up call before graph capture")
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[device] = ws
     return ws
@@ -105,7 +110,7 @@ def paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     max_blocks = block_tables.shape[1]
     lib = _lib.load()
     nbytes = lib.nva_paged_decode_workspace_bytes(b, hq, dh, max(max_blocks, 1))
-    ws = _decode_workspace(q.device, nbytes, torch.cuda.is_current_stream_capturing())
+    ws = _decode_workspace(q.device, nbytes)
     rc = lib.nva_paged_decode_attn(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                    block_tables.data_ptr(), block_tables.stride(0), max_blocks,
                                    context_lens.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),

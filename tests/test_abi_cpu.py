@@ -66,7 +66,9 @@ def test_store_kvcache_validation():
 def test_decode_validation_and_workspace_size():
     lib = _lib.load()
     ws = lib.nva_paged_decode_workspace_bytes
-    assert ws(64, 16, 128, 8) == 64 * 8 * 16 * 130 * 4
+    # prefix sums (256-byte aligned) + (2048 workers * min(heads, 8) + batch * heads) partial rows of 130 floats
+    assert ws(64, 16, 128, 8) == 512 + (2048 * 8 + 64 * 16) * 130 * 4
+    assert ws(3, 2, 128, 1) == 256 + (2048 * 2 + 3 * 2) * 130 * 4
     assert ws(0, 16, 128, 8) == 0
     f = lib.nva_paged_decode_attn
     ok = dict(q=A, qs=2048, kc=A, vc=A, bt=A, bts=8, mb=8, cl=A, out=A, ws=A, wsb=ws(4, 16, 128, 8),
