@@ -5,6 +5,7 @@
 
 A "step" is one pass of the selected workload over one batch of synthetic input that is
 already resident in HBM.  Workloads (shapes are the BASELINE.json configs):
+    e2e       (default) generate() over 256 requests on a Qwen3-0.6B-architecture model (config 4)
     decode    paged decode attention, batch 64, 16/8 heads, ctx U[100,2048]       (config 2)
     scatter   store_kvcache, 4096 tokens into 512 blocks x 256 slots              (config 1)
     prefill   causal varlen prefill, 16 sequences, half with cached prefix        (config 3)
@@ -215,8 +216,83 @@ def bench_sampler(args, dev):
     return result, cpu
 
 
-WORKLOADS = {"decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
-DEFAULT_STEPS = {"decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
+def e2e_workload(num_seqs=256, max_input_len=1024, max_output_len=1024, vocab=151936, seed=0):
+    """The request mix of the reference's bench.py:9-18, ids uniform over the whole vocabulary."""
+    import random
+    from nanovllm_amd.engine import SamplingParams
+    rng = random.Random(seed)
+    prompts = [[rng.randint(0, vocab - 1) for _ in range(rng.randint(100, max_input_len))] for _ in range(num_seqs)]
+    params = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=rng.randint(100, max_output_len))
+              for _ in range(num_seqs)]
+    return prompts, params
+
+
+def bench_e2e(args, dev):
+    """Qwen3-0.6B architecture, random weights, 256 requests, hipGraph decode: output tok/s."""
+    import torch
+    import nanovllm_amd as nva
+    from nanovllm_amd.engine import SamplingParams, qwen3_0_6b
+    from nanovllm_amd.engine.llm import LLM
+    model = qwen3_0_6b()
+    llm = LLM(model, enforce_eager=args.eager, max_model_len=4096, num_kvcache_blocks=4096)
+    prompts, params = e2e_workload(num_seqs=args.requests, max_output_len=args.max_output_len)
+    total_out = sum(p.max_tokens for p in params)
+    llm.generate([[1, 2, 3, 4]], SamplingParams(max_tokens=8, ignore_eos=True))     # reference warm-up call
+    for _ in range(args.warmup):
+        llm.generate(prompts[:32], params[:32])
+    for k in llm.stats:
+        llm.stats[k] = 0
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        outs = llm.generate(prompts, params)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert all(len(o["token_ids"]) == p.max_tokens for o, p in zip(outs, params))
+    tok_s = total_out * args.steps / dt
+
+    # roofline of the dominant kernel (paged decode attention) at this workload's own decode
+    # shape: 256 running sequences whose context lengths are prompt + half of the output, read
+    # through each of the 28 layers' caches in turn (7.5 GB apart, so nothing is cache-resident)
+    from nanovllm_amd import synthetic
+    g = torch.Generator().manual_seed(1)
+    full_prompts, full_params = e2e_workload()
+    ctx = torch.tensor([len(p) + sp.max_tokens // 2 for p, sp in zip(full_prompts, full_params)], dtype=torch.int32)
+    tables = synthetic.decode_tables(ctx.tolist(), llm.config.num_kvcache_blocks, g, width=16).to(dev)
+    ctx_d = ctx.to(dev)
+    q = torch.randn(256, model.num_attention_heads, model.head_dim, device=dev).to(torch.bfloat16)
+    out = torch.empty(256, 1, model.num_attention_heads, model.head_dim, dtype=torch.bfloat16, device=dev)
+    layers = [m for m in llm.model_runner.model.modules() if isinstance(m, nva.Attention)]
+    fns = [lambda a=a: nva.paged_decode_attention(q, a.k_cache, a.v_cache, ctx_d, tables, a.scale, out=out)
+           for a in layers]
+    reps = 5 * len(fns)
+    ms = _event_time_ms(fns, reps, len(fns)) / reps
+    alg = int(ctx.sum()) * model.num_key_value_heads * model.head_dim * 2 * 2 + 2 * q.numel() * 2
+    gbps = alg / (ms * 1e-3) / 1e9
+    st = llm.stats
+    result = {
+        "metric": "output tok/s, Qwen3-0.6B bench shape; decode-attn HBM GB/s vs ~8 TB/s",
+        "value": round(tok_s, 1), "unit": "tok/s", "ms_per_step": round(dt / args.steps * 1e3, 2),
+        "config": {"workload": "e2e generate: Qwen3-0.6B architecture (28 layers, hidden 1024, 16q/8kv heads x 128, "
+                               "MLP 3072, vocab 151936, random bf16 weights), 256 requests, prompt and output lengths "
+                               "U[100,1024], temperature 0.6, ignore_eos, " + ("eager" if args.eager else "hipGraph decode"),
+                   "requests": 256, "output_tokens": total_out, "engine_steps_per_pass": (st["prefill_steps"] + st["decode_steps"]) // args.steps,
+                   "prefill_s_per_pass": round(st["prefill_s"] / args.steps, 3), "decode_s_per_pass": round(st["decode_s"] / args.steps, 3)},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "decode_stream_kernel<2> + decode_merge_kernel<2> (paged decode attention, batch 256, "
+                               "mean ctx %d)" % int(ctx.float().mean()),
+                     "algorithmic_bytes_per_launch": alg, "us_per_launch": round(ms * 1e3, 2)},
+    }
+
+    def cpu():
+        from oracle import engine_cpu
+        return engine_cpu.baseline(model, prompts, params)
+    return result, cpu
+
+
+WORKLOADS = {"e2e": bench_e2e, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
+DEFAULT_STEPS = {"e2e": 1, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
 
 
 def main():
@@ -224,7 +300,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="decode")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="e2e")
+    ap.add_argument("--eager", action="store_true", help="e2e only: no hipGraph decode")
+    ap.add_argument("--requests", type=int, default=256, help="e2e only: number of requests (profiling runs)")
+    ap.add_argument("--max-output-len", type=int, default=1024, help="e2e only: cap on output lengths (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -233,7 +312,7 @@ def main():
     if args.steps is None:
         args.steps = DEFAULT_STEPS[args.workload]
     if args.warmup is None:
-        args.warmup = max(3, args.steps // 10)
+        args.warmup = 1 if args.workload == "e2e" else max(3, args.steps // 10)
 
     import torch
     if not torch.cuda.is_available():

@@ -144,6 +144,46 @@ int nva_sample(const void *logits, int64_t logits_row_stride,
                void *workspace, size_t workspace_bytes,
                int32_t batch, int32_t vocab, void *stream);
 
+/*
+ * ---- steps either side of the hot path (the callers' element-wise glue) ----------------
+ *
+ * RMSNorm, optionally fused with the residual add.  Replaces RMSNorm.rms_forward /
+ * add_rms_forward (nanovllm/layers/layernorm.py:16-40).
+ *   residual == NULL: out = bf16(x * rsqrt(mean(x^2) + eps)) * weight
+ *   otherwise:        s = x + residual (fp32); residual_out = bf16(s);
+ *                     out = bf16(s * rsqrt(mean(s^2) + eps)) * weight
+ * x / residual: bf16 [rows, hidden] with row strides in elements; weight bf16 [hidden];
+ * out / residual_out: bf16 [rows, hidden] dense.  hidden % 8 == 0, hidden <= 4096.
+ */
+int nva_rms_norm(const void *x, int64_t x_row_stride,
+                 const void *residual, int64_t residual_row_stride,
+                 const void *weight, void *out, void *residual_out,
+                 int32_t rows, int32_t hidden, float eps, void *stream);
+
+/*
+ * Per-head RMSNorm of q and k followed by the neox rotary embedding.  Replaces the q_norm /
+ * k_norm / rotary_emb sequence of Qwen3Attention.forward (nanovllm/models/qwen3.py:76-79;
+ * nanovllm/layers/rotary_embedding.py:6-48).
+ * qkv: bf16 [n_tokens, (num_heads + 2*num_kv_heads) * head_dim], row stride in elements
+ * (q heads, then k heads, then v heads; v is left untouched).  positions: int64 [n_tokens].
+ * q_weight / k_weight: bf16 [head_dim].  rope_cache: fp32 [max_position, head_dim], cos in
+ * the first half of a row, sin in the second.  q_out: bf16 [n_tokens, num_heads, head_dim],
+ * k_out: bf16 [n_tokens, num_kv_heads, head_dim], both dense.  head_dim must be 128.
+ */
+int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const int64_t *positions,
+                     const void *q_weight, const void *k_weight, const float *rope_cache,
+                     void *q_out, void *k_out,
+                     int32_t n_tokens, int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
+                     float eps, void *stream);
+
+/*
+ * SwiGLU gate.  Replaces SiluAndMul.forward (nanovllm/layers/activation.py:11-14):
+ * out[r, i] = bf16(silu(x[r, i])) * x[r, inter + i].
+ * x: bf16 [rows, 2*inter] (row stride in elements), out: bf16 [rows, inter] dense, inter % 8 == 0.
+ */
+int nva_silu_and_mul(const void *x, int64_t x_row_stride, void *out,
+                     int32_t rows, int32_t inter, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,185 @@
+// Fused element-wise steps that sit between the GEMMs and the attention hot path.
+//
+// They replace the torch.compile'd fusions of the reference:
+//   rms_norm / add_rms_norm   nanovllm/layers/layernorm.py:16-40
+//   qk_norm_rope              nanovllm/models/qwen3.py:76-79 (per-head RMSNorm of q and k)
+//                             + nanovllm/layers/rotary_embedding.py:6-48 (neox rotation)
+//   silu_and_mul              nanovllm/layers/activation.py:11-14
+// and keep the reference's rounding points: fp32 math, one rounding to bf16 after the
+// normalisation, a bf16 multiply by the bf16 weight, fp32 rotation of the rounded values.
+// All three are pure HBM traffic: every input element is read once, every output written once.
+#include "nva_common.h"
+
+#include <math.h>
+
+namespace nva {
+
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kNormMaxChunks = 8;     // 8 x (64 lanes x 8 elements) = hidden sizes up to 4096
+
+__device__ __forceinline__ float round_bf16(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+
+// One wavefront per row, the row lives in registers between the two passes.
+// residual == nullptr: out = bf16(x * rsqrt(mean(x^2) + eps)) * w
+// else:                s = x + residual (fp32); residual_out = bf16(s); out = bf16(s * rsqrt(mean(s^2) + eps)) * w
+__global__ __launch_bounds__(256) void rms_norm_kernel(
+    const bf16_t *__restrict__ x, int64_t x_stride, const bf16_t *__restrict__ residual, int64_t res_stride,
+    const bf16_t *__restrict__ weight, bf16_t *__restrict__ out, bf16_t *__restrict__ residual_out,
+    int32_t rows, int32_t hidden, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const bf16_t *xr = x + static_cast<int64_t>(row) * x_stride;
+    const bf16_t *rr = residual ? residual + static_cast<int64_t>(row) * res_stride : nullptr;
+    float v[kNormMaxChunks][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < kNormMaxChunks; ++c) {
+        const int e = c * 512 + lane * 8;
+        if (e < hidden) {
+            const uint4 xv = *reinterpret_cast<const uint4 *>(xr + e);
+            unpack8(xv, v[c]);
+            if (rr) {
+                const uint4 rv = *reinterpret_cast<const uint4 *>(rr + e);
+                float rf[8];
+                unpack8(rv, rf);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[c][i] += rf[i];
+                uint4 ro;
+                ro.x = pack_bf16x2(v[c][0], v[c][1]); ro.y = pack_bf16x2(v[c][2], v[c][3]);
+                ro.z = pack_bf16x2(v[c][4], v[c][5]); ro.w = pack_bf16x2(v[c][6], v[c][7]);
+                *reinterpret_cast<uint4 *>(residual_out + static_cast<int64_t>(row) * hidden + e) = ro;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = fmaf(v[c][i], v[c][i], ss);
+        }
+    }
+    ss = wave_sum(ss);
+    const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+#pragma unroll
+    for (int c = 0; c < kNormMaxChunks; ++c) {
+        const int e = c * 512 + lane * 8;
+        if (e < hidden) {
+            const uint4 wv = *reinterpret_cast<const uint4 *>(weight + e);
+            float wf[8], y[8];
+            unpack8(wv, wf);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = round_bf16(v[c][i] * inv) * wf[i];
+            uint4 o;
+            o.x = pack_bf16x2(y[0], y[1]); o.y = pack_bf16x2(y[2], y[3]);
+            o.z = pack_bf16x2(y[4], y[5]); o.w = pack_bf16x2(y[6], y[7]);
+            *reinterpret_cast<uint4 *>(out + static_cast<int64_t>(row) * hidden + e) = o;
+        }
+    }
+}
+
+// One wavefront per (token, head) row of 128 elements; lane l holds elements l and l + 64,
+// which are exactly the pair the neox rotation mixes.  Heads [0, hq) are queries, [hq, hq+hkv)
+// keys; values are not touched (the attention layer reads them in place).
+__global__ __launch_bounds__(256) void qk_norm_rope_kernel(
+    const bf16_t *__restrict__ qkv, int64_t row_stride, const int64_t *__restrict__ positions,
+    const bf16_t *__restrict__ q_weight, const bf16_t *__restrict__ k_weight,
+    const float *__restrict__ rope_cache, bf16_t *__restrict__ q_out, bf16_t *__restrict__ k_out,
+    int64_t n_rows, int32_t hq, int32_t hkv, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (r >= n_rows) return;
+    const int heads = hq + hkv;
+    const int64_t tok = r / heads;
+    const int head = static_cast<int>(r % heads);
+    const bool is_q = head < hq;
+    const bf16_t *src = qkv + tok * row_stride + head * kHeadDim;     // q heads then k heads are adjacent
+    const bf16_t *w = is_q ? q_weight : k_weight;
+    const float x1 = bf16_to_f32(src[lane]);
+    const float x2 = bf16_to_f32(src[lane + 64]);
+    const float ss = wave_sum(fmaf(x1, x1, x2 * x2));
+    const float inv = rsqrtf(ss * (1.0f / kHeadDim) + eps);
+    const float y1 = round_bf16(round_bf16(x1 * inv) * bf16_to_f32(w[lane]));
+    const float y2 = round_bf16(round_bf16(x2 * inv) * bf16_to_f32(w[lane + 64]));
+    const float *cs = rope_cache + positions[tok] * kHeadDim;
+    const float c = cs[lane], s = cs[lane + 64];
+    bf16_t *dst = is_q ? q_out + (tok * hq + head) * kHeadDim : k_out + (tok * hkv + (head - hq)) * kHeadDim;
+    dst[lane] = f32_to_bf16(y1 * c - y2 * s);
+    dst[lane + 64] = f32_to_bf16(y2 * c + y1 * s);
+}
+
+// out[r, i] = bf16(silu(x[r, i])) * x[r, inter + i], 8 elements per lane
+__global__ __launch_bounds__(256) void silu_and_mul_kernel(const bf16_t *__restrict__ x, int64_t row_stride,
+                                                           bf16_t *__restrict__ out, int64_t total_chunks,
+                                                           int32_t chunks_per_row, int32_t inter) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total_chunks) return;
+    const int64_t row = idx / chunks_per_row;
+    const int e = static_cast<int>(idx % chunks_per_row) * 8;
+    const bf16_t *xr = x + row * row_stride;
+    float g[8], u[8];
+    unpack8(*reinterpret_cast<const uint4 *>(xr + e), g);
+    unpack8(*reinterpret_cast<const uint4 *>(xr + inter + e), u);
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = round_bf16(g[i] / (1.0f + expf(-g[i]))) * u[i];
+    uint4 o;
+    o.x = pack_bf16x2(y[0], y[1]); o.y = pack_bf16x2(y[2], y[3]);
+    o.z = pack_bf16x2(y[4], y[5]); o.w = pack_bf16x2(y[6], y[7]);
+    *reinterpret_cast<uint4 *>(out + row * inter + e) = o;
+}
+
+}  // namespace nva
+
+extern "C" int nva_rms_norm(const void *x, int64_t x_row_stride, const void *residual, int64_t residual_row_stride,
+                            const void *weight, void *out, void *residual_out, int32_t rows, int32_t hidden,
+                            float eps, void *stream) {
+    using namespace nva;
+    if (rows < 0 || hidden <= 0) return NVA_ERR_BAD_SHAPE;
+    if (hidden % 8 != 0 || hidden > kNormMaxChunks * 512) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+    if (rows == 0) return NVA_OK;
+    if (!x || !weight || !out) return NVA_ERR_NULL_POINTER;
+    if (residual && !residual_out) return NVA_ERR_NULL_POINTER;
+    if (x_row_stride < hidden || x_row_stride % 8 != 0) return NVA_ERR_BAD_STRIDE;
+    if (residual && (residual_row_stride < hidden || residual_row_stride % 8 != 0)) return NVA_ERR_BAD_STRIDE;
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(out) || (residual && (!aligned16(residual) || !aligned16(residual_out))))
+        return NVA_ERR_MISALIGNED;
+    hipLaunchKernelGGL(rms_norm_kernel, dim3((rows + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const bf16_t *>(x), x_row_stride, static_cast<const bf16_t *>(residual),
+                       residual_row_stride, static_cast<const bf16_t *>(weight), static_cast<bf16_t *>(out),
+                       static_cast<bf16_t *>(residual_out), rows, hidden, eps);
+    return launch_status();
+}
+
+extern "C" int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const int64_t *positions,
+                                const void *q_weight, const void *k_weight, const float *rope_cache,
+                                void *q_out, void *k_out, int32_t n_tokens, int32_t num_heads,
+                                int32_t num_kv_heads, int32_t head_dim, float eps, void *stream) {
+    using namespace nva;
+    if (n_tokens < 0 || num_heads <= 0 || num_kv_heads <= 0) return NVA_ERR_BAD_SHAPE;
+    if (head_dim != kHeadDim) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+    if (n_tokens == 0) return NVA_OK;
+    if (!qkv || !positions || !q_weight || !k_weight || !rope_cache || !q_out || !k_out) return NVA_ERR_NULL_POINTER;
+    if (qkv_row_stride < static_cast<int64_t>(num_heads + 2 * num_kv_heads) * head_dim) return NVA_ERR_BAD_STRIDE;
+    const int64_t n_rows = static_cast<int64_t>(n_tokens) * (num_heads + num_kv_heads);
+    if ((n_rows + 3) / 4 > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(qk_norm_rope_kernel, dim3(static_cast<uint32_t>((n_rows + 3) / 4)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const bf16_t *>(qkv), qkv_row_stride, positions,
+                       static_cast<const bf16_t *>(q_weight), static_cast<const bf16_t *>(k_weight), rope_cache,
+                       static_cast<bf16_t *>(q_out), static_cast<bf16_t *>(k_out), n_rows, num_heads, num_kv_heads, eps);
+    return launch_status();
+}
+
+extern "C" int nva_silu_and_mul(const void *x, int64_t x_row_stride, void *out, int32_t rows, int32_t inter,
+                                void *stream) {
+    using namespace nva;
+    if (rows < 0 || inter <= 0) return NVA_ERR_BAD_SHAPE;
+    if (inter % 8 != 0) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+    if (rows == 0) return NVA_OK;
+    if (!x || !out) return NVA_ERR_NULL_POINTER;
+    if (x_row_stride < 2 * static_cast<int64_t>(inter) || x_row_stride % 8 != 0) return NVA_ERR_BAD_STRIDE;
+    if (!aligned16(x) || !aligned16(out)) return NVA_ERR_MISALIGNED;
+    const int32_t chunks_per_row = inter / 8;
+    const int64_t total = static_cast<int64_t>(rows) * chunks_per_row;
+    if ((total + 255) / 256 > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(silu_and_mul_kernel, dim3(static_cast<uint32_t>((total + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const bf16_t *>(x), x_row_stride,
+                       static_cast<bf16_t *>(out), total, chunks_per_row, inter);
+    return launch_status();
+}

@@ -1,0 +1,80 @@
+"""Element-wise / normalisation glue between the GEMMs of a Qwen3 layer, on the GPU.
+
+Thin wrappers over the fused C-ABI kernels (csrc/glue.hip) that replace the reference's
+torch.compile'd fusions: nanovllm/layers/layernorm.py:16-40, rotary_embedding.py:6-48 with
+the per-head q/k norms of nanovllm/models/qwen3.py:76-79, and activation.py:11-14.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+_BF16 = torch.bfloat16
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """``bf16(x * rsqrt(mean(x^2) + eps)) * weight`` over the last dim of a 2-D tensor."""
+    assert x.dim() == 2 and x.dtype == _BF16 and x.stride(1) == 1 and x.is_cuda
+    out = torch.empty((x.shape[0], x.shape[1]), dtype=_BF16, device=x.device)
+    rc = _lib.load().nva_rms_norm(x.data_ptr(), x.stride(0), None, 0, weight.data_ptr(), out.data_ptr(), None,
+                                  x.shape[0], x.shape[1], float(eps), _stream())
+    _lib.check(rc, "nva_rms_norm")
+    return out
+
+
+def add_rms_norm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float):
+    """Returns ``(normed(x + residual), bf16(x + residual))``."""
+    assert x.dim() == 2 and x.dtype == _BF16 and x.stride(1) == 1 and x.is_cuda
+    assert residual.shape == x.shape and residual.dtype == _BF16 and residual.stride(1) == 1
+    out = torch.empty((x.shape[0], x.shape[1]), dtype=_BF16, device=x.device)
+    res_out = torch.empty_like(out)
+    rc = _lib.load().nva_rms_norm(x.data_ptr(), x.stride(0), residual.data_ptr(), residual.stride(0),
+                                  weight.data_ptr(), out.data_ptr(), res_out.data_ptr(),
+                                  x.shape[0], x.shape[1], float(eps), _stream())
+    _lib.check(rc, "nva_rms_norm")
+    return out, res_out
+
+
+def build_rope_cache(head_dim: int, max_position: int, base: float, device) -> torch.Tensor:
+    """``[max_position, head_dim]`` fp32: cos in the first half of a row, sin in the second
+    (the table of nanovllm/layers/rotary_embedding.py:28-35)."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float, device=device) / head_dim))
+    t = torch.arange(max_position, dtype=torch.float, device=device)
+    freqs = torch.outer(t, inv_freq)
+    return torch.cat((freqs.cos(), freqs.sin()), dim=-1).contiguous()
+
+
+def qk_norm_rope(qkv: torch.Tensor, positions: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor,
+                 rope_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, eps: float):
+    """Per-head RMSNorm of q and k, then the rotary embedding.
+
+    Returns ``(q, k, v)`` with q, k fresh contiguous ``[N, H, Dh]`` tensors and v a strided
+    view into ``qkv`` -- the layouts nanovllm/models/qwen3.py:74-79 hands to the attention layer.
+    """
+    n = qkv.shape[0]
+    assert qkv.dim() == 2 and qkv.dtype == _BF16 and qkv.stride(1) == 1 and qkv.is_cuda
+    assert qkv.shape[1] == (num_heads + 2 * num_kv_heads) * head_dim
+    assert positions.dtype == torch.int64 and positions.numel() == n and positions.is_contiguous()
+    assert rope_cache.dtype == torch.float32 and rope_cache.is_contiguous() and rope_cache.shape[1] == head_dim
+    q = torch.empty((n, num_heads, head_dim), dtype=_BF16, device=qkv.device)
+    k = torch.empty((n, num_kv_heads, head_dim), dtype=_BF16, device=qkv.device)
+    rc = _lib.load().nva_qk_norm_rope(qkv.data_ptr(), qkv.stride(0), positions.data_ptr(), q_weight.data_ptr(),
+                                      k_weight.data_ptr(), rope_cache.data_ptr(), q.data_ptr(), k.data_ptr(),
+                                      n, num_heads, num_kv_heads, head_dim, float(eps), _stream())
+    _lib.check(rc, "nva_qk_norm_rope")
+    v = qkv[:, (num_heads + num_kv_heads) * head_dim:].view(n, num_kv_heads, head_dim)
+    return q, k, v
+
+
+def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
+    assert x.dim() == 2 and x.dtype == _BF16 and x.stride(1) == 1 and x.shape[1] % 2 == 0 and x.is_cuda
+    inter = x.shape[1] // 2
+    out = torch.empty((x.shape[0], inter), dtype=_BF16, device=x.device)
+    rc = _lib.load().nva_silu_and_mul(x.data_ptr(), x.stride(0), out.data_ptr(), x.shape[0], inter, _stream())
+    _lib.check(rc, "nva_silu_and_mul")
+    return out

@@ -1,0 +1,216 @@
+"""Builds the per-step device tensors, owns the KV cache and the decode graphs, runs the model.
+
+Single-GPU counterpart of nanovllm/engine/model_runner.py: ``prepare_prefill`` /
+``prepare_decode`` reproduce the reference's input layouts (:126-179), ``allocate_kv_cache``
+its cache layout ``[2, layers, num_blocks, 256, Hkv, Dh]`` (:100-117) and ``capture_graphs``
+its static-buffer graph replay per batch-size bucket (:215-250).  Host tensors are built
+with numpy into pinned staging buffers instead of Python lists.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import numpy as np
+import torch
+
+from ..context import get_context, reset_context, set_context
+from ..sampler import Sampler
+from .config import EngineConfig
+from .model import Qwen3ForCausalLM
+from .sequence import Sequence
+
+
+def build_block_tables(seqs: List[Sequence]) -> np.ndarray:
+    """``[len(seqs), widest table]`` int32, rows padded with -1 (model_runner.py:119-124)."""
+    width = max(len(s.block_table) for s in seqs)
+    table = np.full((len(seqs), width), -1, dtype=np.int32)
+    for i, s in enumerate(seqs):
+        table[i, : len(s.block_table)] = s.block_table
+    return table
+
+
+def build_prefill_inputs(seqs: List[Sequence], block_size: int) -> dict:
+    """Host-side inputs of a prefill step (nanovllm/engine/model_runner.py:126-160).
+
+    Only the uncached tail ``[num_cached_tokens, len)`` of every sequence is run: those are
+    the input ids, positions and query lengths; key lengths are the full lengths.  The slot
+    of position p is ``block_table[p // bs] * bs + p % bs``.  ``block_tables`` is present only
+    when some sequence has cached tokens.
+    """
+    ids, pos, slots = [], [], []
+    cu_q, cu_k = [0], [0]
+    max_q = max_k = 0
+    for s in seqs:
+        n, cached = len(s), s.num_cached_tokens
+        ids.append(np.asarray(s.token_ids[cached:], dtype=np.int64))
+        p = np.arange(cached, n, dtype=np.int64)
+        pos.append(p)
+        cu_q.append(cu_q[-1] + n - cached)
+        cu_k.append(cu_k[-1] + n)
+        max_q, max_k = max(max_q, n - cached), max(max_k, n)
+        if s.block_table:                                         # empty during warm-up
+            table = np.asarray(s.block_table, dtype=np.int64)
+            slots.append(table[p // block_size] * block_size + p % block_size)
+    return dict(
+        input_ids=np.concatenate(ids), positions=np.concatenate(pos),
+        cu_seqlens_q=np.asarray(cu_q, dtype=np.int32), cu_seqlens_k=np.asarray(cu_k, dtype=np.int32),
+        max_seqlen_q=max_q, max_seqlen_k=max_k,
+        slot_mapping=(np.concatenate(slots) if slots else np.empty(0, np.int64)).astype(np.int32),
+        block_tables=build_block_tables(seqs) if cu_k[-1] > cu_q[-1] else None)
+
+
+def build_decode_inputs(seqs: List[Sequence], block_size: int) -> dict:
+    """Host-side inputs of a decode step (nanovllm/engine/model_runner.py:162-179): the last
+    token of every sequence at position len-1, written to the last block of its table."""
+    n = len(seqs)
+    ids = np.fromiter((s.token_ids[-1] for s in seqs), dtype=np.int64, count=n)
+    lens = np.fromiter((len(s.token_ids) for s in seqs), dtype=np.int64, count=n)
+    last_blk = np.fromiter((s.block_table[-1] for s in seqs), dtype=np.int64, count=n)
+    return dict(input_ids=ids, positions=lens - 1, context_lens=lens.astype(np.int32),
+                slot_mapping=(last_blk * block_size + (lens - 1) % block_size).astype(np.int32),
+                block_tables=build_block_tables(seqs))
+
+
+class ModelRunner:
+
+    def __init__(self, config: EngineConfig, device: str = "cuda:0"):
+        self.config = config
+        self.cfg = config.hf_config
+        self.block_size = config.kvcache_block_size
+        self.enforce_eager = config.enforce_eager
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        prev = torch.get_default_dtype()
+        torch.set_default_dtype(torch.bfloat16)
+        try:
+            with torch.device(self.device):
+                self.model = Qwen3ForCausalLM(self.cfg, config.max_model_len, self.device, config.seed)
+        finally:
+            torch.set_default_dtype(prev)
+        self.model.eval()
+        self.sampler = Sampler(seed=config.seed)
+        self.max_table_width = -(-config.max_model_len // self.block_size)
+        self.graphs = {}
+        self.graph_bs: List[int] = []
+        with torch.inference_mode():
+            self.warmup_model()
+            self.allocate_kv_cache()
+            if not self.enforce_eager:
+                self.capture_graphs()
+
+    # ---- set-up ------------------------------------------------------------------------------
+    def warmup_model(self) -> None:
+        """One prefill of the largest admissible batch, cache not yet allocated: the attention
+        layers skip the scatter and run packed (non-paged) prefill, which is also what sizes the
+        activation peak used to carve the KV cache out of free memory."""
+        torch.cuda.empty_cache()
+        torch.cuda.reset_peak_memory_stats()
+        cfg = self.config
+        num_seqs = max(1, min(cfg.max_num_batched_tokens // cfg.max_model_len, cfg.max_num_seqs))
+        seqs = [Sequence([0] * cfg.max_model_len) for _ in range(num_seqs)]
+        self.run(seqs, True)
+        torch.cuda.empty_cache()
+
+    def allocate_kv_cache(self) -> None:
+        cfg, m = self.config, self.cfg
+        block_bytes = 2 * m.num_hidden_layers * self.block_size * m.num_key_value_heads * m.head_dim * 2
+        if cfg.num_kvcache_blocks <= 0:
+            free, total = torch.cuda.mem_get_info()
+            stats = torch.cuda.memory_stats()
+            peak, current = stats["allocated_bytes.all.peak"], stats["allocated_bytes.all.current"]
+            budget = int(total * cfg.gpu_memory_utilization) - (total - free) - peak + current
+            cfg.num_kvcache_blocks = budget // block_bytes
+        assert cfg.num_kvcache_blocks > 0, "no memory left for the KV cache"
+        self.kv_cache = torch.empty(2, m.num_hidden_layers, cfg.num_kvcache_blocks, self.block_size,
+                                    m.num_key_value_heads, m.head_dim, dtype=torch.bfloat16, device=self.device)
+        layer_id = 0
+        for module in self.model.modules():
+            if hasattr(module, "k_cache") and hasattr(module, "v_cache"):
+                module.k_cache = self.kv_cache[0, layer_id]
+                module.v_cache = self.kv_cache[1, layer_id]
+                layer_id += 1
+        assert layer_id == m.num_hidden_layers
+
+    # ---- host -> device inputs -----------------------------------------------------------------
+    def _to_device(self, array: np.ndarray, dtype: torch.dtype) -> torch.Tensor:
+        t = torch.from_numpy(np.ascontiguousarray(array)).to(dtype)
+        return t.pin_memory().to(self.device, non_blocking=True)
+
+    def prepare_block_tables(self, seqs: List[Sequence]) -> torch.Tensor:
+        return self._to_device(build_block_tables(seqs), torch.int32)
+
+    def prepare_prefill(self, seqs: List[Sequence]):
+        h = build_prefill_inputs(seqs, self.block_size)
+        block_tables = self._to_device(h["block_tables"], torch.int32) if h["block_tables"] is not None else None
+        set_context(True, self._to_device(h["cu_seqlens_q"], torch.int32), self._to_device(h["cu_seqlens_k"], torch.int32),
+                    h["max_seqlen_q"], h["max_seqlen_k"], self._to_device(h["slot_mapping"], torch.int32), None,
+                    block_tables)
+        return self._to_device(h["input_ids"], torch.int64), self._to_device(h["positions"], torch.int64)
+
+    def prepare_decode(self, seqs: List[Sequence]):
+        h = build_decode_inputs(seqs, self.block_size)
+        set_context(False, slot_mapping=self._to_device(h["slot_mapping"], torch.int32),
+                    context_lens=self._to_device(h["context_lens"], torch.int32),
+                    block_tables=self._to_device(h["block_tables"], torch.int32))
+        return self._to_device(h["input_ids"], torch.int64), self._to_device(h["positions"], torch.int64)
+
+    def prepare_sample(self, seqs: List[Sequence]) -> torch.Tensor:
+        return self._to_device(np.fromiter((s.temperature for s in seqs), dtype=np.float32, count=len(seqs)),
+                               torch.float32)
+
+    # ---- execution -----------------------------------------------------------------------------
+    @torch.inference_mode()
+    def run_model(self, input_ids: torch.Tensor, positions: torch.Tensor, is_prefill: bool) -> torch.Tensor:
+        bs = input_ids.size(0)
+        if is_prefill or self.enforce_eager or not self.graph_bs or bs > self.graph_bs[-1]:
+            return self.model.compute_logits(self.model(input_ids, positions))
+        ctx = get_context()
+        bucket = next(x for x in self.graph_bs if x >= bs)
+        gv = self.graph_vars
+        gv["input_ids"][:bs] = input_ids
+        gv["positions"][:bs] = positions
+        gv["slot_mapping"].fill_(-1)                              # padded rows store nothing ...
+        gv["slot_mapping"][:bs] = ctx.slot_mapping
+        gv["context_lens"].zero_()                                # ... and attend over nothing
+        gv["context_lens"][:bs] = ctx.context_lens
+        gv["block_tables"][:bs, : ctx.block_tables.size(1)] = ctx.block_tables   # stale columns stay: never read
+        self.graphs[bucket].replay()
+        return self.model.compute_logits(gv["outputs"][:bs])
+
+    def run(self, seqs: List[Sequence], is_prefill: bool) -> List[int]:
+        with torch.inference_mode():
+            input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
+            temperatures = self.prepare_sample(seqs)
+            logits = self.run_model(input_ids, positions, is_prefill)
+            tokens = self.sampler(logits, temperatures).tolist()   # the one device->host sync per step
+        reset_context()
+        return tokens
+
+    @torch.inference_mode()
+    def capture_graphs(self) -> None:
+        cfg = self.config
+        max_bs = min(cfg.max_num_seqs, 512)
+        dev = self.device
+        input_ids = torch.zeros(max_bs, dtype=torch.int64, device=dev)
+        positions = torch.zeros(max_bs, dtype=torch.int64, device=dev)
+        slot_mapping = torch.zeros(max_bs, dtype=torch.int32, device=dev)
+        context_lens = torch.zeros(max_bs, dtype=torch.int32, device=dev)
+        block_tables = torch.zeros(max_bs, self.max_table_width, dtype=torch.int32, device=dev)
+        outputs = torch.zeros(max_bs, self.cfg.hidden_size, dtype=torch.bfloat16, device=dev)
+        self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))
+        pool = None
+        for bs in reversed(self.graph_bs):
+            graph = torch.cuda.CUDAGraph()
+            set_context(False, slot_mapping=slot_mapping[:bs], context_lens=context_lens[:bs],
+                        block_tables=block_tables[:bs])
+            outputs[:bs] = self.model(input_ids[:bs], positions[:bs])        # eager warm-up (sizes workspaces)
+            with torch.cuda.graph(graph, pool):
+                outputs[:bs] = self.model(input_ids[:bs], positions[:bs])
+            if pool is None:
+                pool = graph.pool()
+            self.graphs[bs] = graph
+            torch.cuda.synchronize()
+            reset_context()
+        self.graph_pool = pool
+        self.graph_vars = dict(input_ids=input_ids, positions=positions, slot_mapping=slot_mapping,
+                               context_lens=context_lens, block_tables=block_tables, outputs=outputs)

@@ -1,0 +1,80 @@
+"""Fused glue kernels (RMSNorm, q/k-norm + rotary, SwiGLU gate) against oracle/glue.py.
+
+The kernels keep the reference's rounding points, so results agree to the last bf16 bit
+except where a different fp32 summation order moves a value across a rounding boundary:
+the tests allow one bf16 ulp on a small fraction of the elements (two on a handful)."""
+import pytest
+import torch
+
+from oracle import glue
+from nanovllm_amd.engine import layers
+
+pytestmark = pytest.mark.gpu
+
+
+def assert_bf16_close(got, want, what, max_frac=0.02):
+    got, want = got.detach().float().cpu(), want.detach().float().cpu()
+    assert got.shape == want.shape, (got.shape, want.shape)
+    assert torch.isfinite(got).all()
+    ulp = want.abs().clamp_min(1e-30) * 2.0 ** -7          # one bf16 step at the value's magnitude
+    diff = (got - want).abs()
+    # the value is rounded twice (after the normalisation and after the weight multiply), so a
+    # one-ulp difference of the first rounding can become two ulps at the output
+    assert bool((diff <= ulp * 2.02 + 1e-30).all()), f"{what}: max diff {float(diff.max())} exceeds two bf16 ulps"
+    assert float((diff > ulp * 1.01).float().mean()) <= 1e-4, f"{what}: too many two-ulp differences"
+    frac = float((diff > 0).float().mean())
+    assert frac <= max_frac, f"{what}: {frac:.4f} of the elements differ"
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 1024), (256, 1024), (77, 4096), (5, 128), (3, 1000), (4097, 1024)])
+def test_rms_norm_and_add_rms_norm(dev, rows, hidden):
+    g = torch.Generator().manual_seed(rows + hidden)
+    x = (torch.randn(rows, hidden, generator=g) * 3).to(torch.bfloat16)
+    r = torch.randn(rows, hidden, generator=g).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(torch.bfloat16)
+    out = layers.rms_norm(x.to(dev), w.to(dev), 1e-6)
+    assert_bf16_close(out, glue.rms_norm(x, w, 1e-6), "rms_norm")
+    out2, res2 = layers.add_rms_norm(x.to(dev), r.to(dev), w.to(dev), 1e-6)
+    want, want_res = glue.add_rms_norm(x, r, w, 1e-6)
+    assert torch.equal(res2.cpu().view(torch.int16), want_res.view(torch.int16))     # the sum is exact
+    assert_bf16_close(out2, want, "add_rms_norm")
+
+
+def test_rms_norm_strided_rows(dev):
+    g = torch.Generator().manual_seed(9)
+    wide = torch.randn(16, 2048, generator=g).to(torch.bfloat16)
+    w = torch.ones(1024, dtype=torch.bfloat16)
+    out = layers.rms_norm(wide.to(dev)[:, 512:1536], w.to(dev), 1e-6)
+    assert_bf16_close(out, glue.rms_norm(wide[:, 512:1536], w, 1e-6), "strided")
+
+
+@pytest.mark.parametrize("n,hq,hkv", [(1, 16, 8), (256, 16, 8), (1000, 32, 8), (3, 4, 1)])
+def test_qk_norm_rope(dev, n, hq, hkv):
+    g = torch.Generator().manual_seed(n)
+    d = 128
+    qkv = torch.randn(n, (hq + 2 * hkv) * d, generator=g).to(torch.bfloat16)
+    qw = (1 + 0.2 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    kw = (1 + 0.2 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    pos = torch.randint(0, 4096, (n,), generator=g)
+    cache = glue.build_rope_cache(d, 4096, 1e6)
+    cache_d = layers.build_rope_cache(d, 4096, 1e6, dev)
+    assert (cache_d.cpu() - cache).abs().max() < 1e-3         # table built on the device: pow() differs in the last ulp and positions up to 4095 amplify it
+    qkv_d = qkv.to(dev)
+    q, k, v = layers.qk_norm_rope(qkv_d, pos.to(dev), qw.to(dev), kw.to(dev), cache.to(dev), hq, hkv, d, 1e-6)
+    wq, wk, wv = glue.qk_norm_rope(qkv, pos, qw, kw, cache, hq, hkv, d, 1e-6)
+    assert q.is_contiguous() and k.is_contiguous()
+    assert v.data_ptr() == qkv_d.data_ptr() + (hq + hkv) * d * 2 and (n == 1 or v.stride(0) == (hq + 2 * hkv) * d)
+    assert torch.equal(v.cpu().view(torch.int16), wv.contiguous().view(torch.int16))
+    # the rotation subtracts nearly equal products: compare against the value scale, not per element
+    for got, want, name in ((q, wq, "q"), (k, wk, "k")):
+        diff = (got.float().cpu() - want.float()).abs()
+        assert float(diff.max()) <= 2.0 ** -6 * float(want.float().abs().max()), name
+        assert float(diff.mean()) <= 1e-3, name
+
+
+@pytest.mark.parametrize("rows,inter", [(1, 3072), (256, 3072), (50, 12288), (7, 8)])
+def test_silu_and_mul(dev, rows, inter):
+    g = torch.Generator().manual_seed(inter)
+    x = (torch.randn(rows, 2 * inter, generator=g) * 2).to(torch.bfloat16)
+    out = layers.silu_and_mul(x.to(dev))
+    assert_bf16_close(out, glue.silu_and_mul(x), "silu_and_mul", max_frac=0.01)
