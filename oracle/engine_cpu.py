@@ -109,7 +109,7 @@ def random_weights(cfg, seed: int = 0) -> Dict[str, torch.Tensor]:
     return w
 
 
-def baseline(cfg, prompts: List[List[int]], params, num_requests: int = 8, max_new_tokens: int = 12,
+def baseline(cfg, prompts: List[List[int]], params, num_requests: int = 16, max_new_tokens: int = 32,
              budget_s: float = 30.0) -> dict:
     """cpu_baseline for the end-to-end workload: the first ``num_requests`` requests of the bench
     mix, outputs capped at ``max_new_tokens``, run through the same scheduler / block manager
