@@ -30,9 +30,10 @@
 // When a worker leaves a (sequence, kv head) pair it either writes the final bf16 rows (it
 // saw all of the pair's stages) or an unnormalised partial (max, sum, o[128]) per query
 // head.  A second, small kernel (decode_merge_kernel) merges the partials of the pairs that
-// were split over several workers; the kernel boundary is the only synchronisation (device
-// wide fences inside the streaming kernel cost far more than the boundary: they flush the
-// L2 of the XCD).
+// were split over several workers; the kernel boundary is the only synchronisation.  (Workers
+// sit on different XCDs, each with its own L2.  An in-kernel "last arriver merges" variant needs
+// device-scope fences, which write back and invalidate the XCD's L2: measured 3x slower for
+// the whole kernel.  Relaxed device-scope atomics without fences returned stale partials.)
 //
 // HBM traffic per sequence and layer: ctx * num_kv_heads * 128 * 2 B for K plus the same for
 // V (4096 B per token at 8 kv heads).  Partials: at most (W + batch*num_kv_heads) * G rows of 520 B.
@@ -90,6 +91,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
 
     // ---- stage-count prefix sums over the batch (every workgroup computes its own copy) -------
     __shared__ int32_t sh_pref[kDecMaxBatch + 1];   // sh_pref[b] = stages of all (sequence < b, head)
+    __shared__ int32_t sh_ctx[kDecMaxBatch];        // context length of sequence b, clipped to the table
     __shared__ __attribute__((aligned(16))) u32x4_t lds[kDecWaves * kWaveLdsChunks];
     if (wave == 0) {
         constexpr int kPer = kDecMaxBatch / kWave;  // 16 sequences per lane
@@ -100,10 +102,10 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
             const int b = lane * kPer + i;
             int c = 0;
             if (b < a.batch) {
-                const int ctx = a.context_lens[b];
-                const int st = ctx > 0 ? (ctx + kStageTok - 1) / kStageTok : 0;
                 // a context that does not fit the table is clipped to it instead of read out of bounds
-                c = min(st, a.max_blocks * kStagesPerBlock) * hkv;
+                const int ctx = min(max(a.context_lens[b], 0), a.max_blocks * kBlockSize);
+                sh_ctx[b] = ctx;
+                c = (ctx + kStageTok - 1) / kStageTok * hkv;
             }
             cnt[i] = c;
             local += c;
@@ -164,10 +166,9 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
 
     // HBM -> registers for stage (bb, gg, ss) of a sequence with nn stages per head.  Token rows
     // are clamped to the last valid row of the stage, so only rows that were written are touched.
-    auto load_stage = [&](int bb, int gg, int ss, int nn, u32x4_t (&kr)[kStageLoads], u32x4_t (&vr)[kStageLoads],
+    auto load_stage = [&](int bb, int gg, int ss, u32x4_t (&kr)[kStageLoads], u32x4_t (&vr)[kStageLoads],
                           u32x4_t (&qr)[4], int &last) __attribute__((always_inline)) {
-        const int ctx = min(a.context_lens[bb], nn * kStageTok);
-        last = min(kStageTok, ctx - ss * kStageTok) - 1;                       // in [0, 31]
+        last = min(kStageTok, sh_ctx[bb] - ss * kStageTok) - 1;                // in [0, 31]
         int32_t blk = a.block_tables[static_cast<int64_t>(bb) * a.bt_row_stride + ss / kStagesPerBlock];
         if (static_cast<uint32_t>(blk) >= static_cast<uint32_t>(a.num_blocks)) {
             blk = 0;                                  // bad table entry: contributes nothing
@@ -207,7 +208,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
 
     u32x4_t kr[kStageLoads], vr[kStageLoads], qr[4];
     int last;
-    load_stage(b, g, s, nst, kr, vr, qr, last);
+    load_stage(b, g, s, kr, vr, qr, last);
 
     for (int64_t x = lo; x < hi; ++x) {
         // ---- registers -> LDS (swizzled) ------------------------------------------------------
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
                     nst = (sh_pref[b + 1] - sh_pref[b]) / hkv;
                 }
             }
-            load_stage(b, g, s, nst, kr, vr, qr, last);
+            load_stage(b, g, s, kr, vr, qr, last);
         }
         __builtin_amdgcn_wave_barrier();
 

@@ -115,3 +115,24 @@ def test_decode_q_as_4d_and_strided(dev):
                                  case.context_lens.to(dev), case.block_tables.to(dev), case.scale)
     torch.cuda.synchronize()
     assert_attn_close(out, _oracle(case), "strided q")
+
+
+def test_decode_partials_are_fresh_across_calls(dev):
+    """Split partials travel between XCDs through memory.  Two different inputs of the same shape
+    use the same partial rows, so a stale read would surface as a mismatch when they alternate."""
+    cases = [synthetic.decode_case(seed=40 + i, batch=24, num_blocks=256, ctx_lo=1500, ctx_hi=1600) for i in range(2)]
+    cases[1].context_lens[:] = cases[0].context_lens            # same stage list, same split, other values
+    cases[1] = synthetic.DecodeCase(cases[1].q, cases[1].k_cache, cases[1].v_cache, cases[0].context_lens,
+                                    cases[0].block_tables, cases[1].scale)
+    dev_in = [(c.q.to(dev), c.k_cache.to(dev), c.v_cache.to(dev), c.context_lens.to(dev), c.block_tables.to(dev))
+              for c in cases]
+    good = []
+    for c, d in zip(cases, dev_in):
+        out = paged_decode_attention(*d, c.scale)
+        torch.cuda.synchronize()
+        assert_attn_close(out, _oracle(c), "alternating")
+        good.append(out.clone())
+    for it in range(300):
+        i = it & 1
+        out = paged_decode_attention(*dev_in[i], cases[i].scale)
+        assert torch.equal(out, good[i]), f"iteration {it}"
