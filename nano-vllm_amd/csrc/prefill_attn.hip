@@ -4,11 +4,16 @@
 // the prefix-cache case where K/V of every sequence are read through the block table.
 //
 // One workgroup of 4 wavefronts per (128-query tile, query head, sequence); wavefront w owns
-// 32 query rows.  Keys are walked in tiles of 64; a K tile and a V tile ([64][128] bf16,
-// rows padded to 272 B) are staged in LDS.  Everything is computed transposed so that a
-// query is a LANE (lane % 32) and keys / output dims live in that lane's registers:
+// 32 query rows.  Keys are walked in tiles of 64.  The K and V tiles ([64][128] bf16 each) are
+// double-buffered in LDS: the global loads of tile t+1 are issued into registers before the
+// arithmetic of tile t and written to the other buffer afterwards, one barrier per tile.
+// Rows keep their 256-byte pitch; the 16-byte chunk index is XOR-swizzled per key (K: by
+// key%16, V: by 4*(key%4)) so that the operand reads below are spread over all banks.
+// Everything is computed transposed so that a query is a LANE (lane % 32) and keys / output
+// dims live in that lane's registers:
 //     S^T = K * Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q^T (registers)
-//     O^T = V^T * P^T    A = V^T gathered from LDS, B = P^T straight from the S^T accumulators
+//     O^T = V^T * P^T    A = V^T through ds_read_b64_tr_b16 (LDS transpose read: 4 keys x 16
+//                        dims -> lane = dim, registers = keys), B = P^T from the S^T registers
 // The softmax state (running max, running sum) is therefore per lane, reductions over keys
 // are in-register, and the only cross-lane step is one exchange between lanes l and l^32,
 // which hold the two key halves of the same query.  The S^T accumulator layout (register i
@@ -25,11 +30,15 @@ namespace nva {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));   // plain vectors: stay in registers
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
 
 constexpr int kPfThreads = 256;
 constexpr int kPfBM = 128;            // queries per workgroup
 constexpr int kPfBN = 64;             // keys per LDS tile
-constexpr int kPfLd = kHeadDim + 8;   // padded LDS row, elements (272 B)
+constexpr int kPfTileChunks = kPfBN * 16;   // 16-byte chunks per K (or V) tile
 
 struct PrefillArgs {
     const bf16_t *q; int64_t q_row_stride;
@@ -43,10 +52,10 @@ struct PrefillArgs {
     float scale_log2e;
 };
 
-__device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 &u) { return __builtin_bit_cast(bf16x8_t, u); }
+__device__ __forceinline__ bf16x8_t as_bf16x8(const u32x4_t &u) { return __builtin_bit_cast(bf16x8_t, u); }
 
 template <bool kPaged>
-__global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillArgs a) {
+__global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const PrefillArgs a) {
     // Workgroups go to the 8 XCDs round-robin by linear id, so the head is the fastest index
     // (every XCD gets the same mix of tiles however ragged the sequences are) and the query
     // tiles run from the last one (most keys, longest) to the first.
@@ -73,7 +82,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillA
     {
         const bf16_t *qp = a.q + static_cast<int64_t>(q0 + qrow_c) * a.q_row_stride + h * kHeadDim + 8 * hh;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) qfrag[s] = as_bf16x8(*reinterpret_cast<const uint4 *>(qp + 16 * s));
+        for (int s = 0; s < 8; ++s) qfrag[s] = as_bf16x8(*reinterpret_cast<const u32x4_t *>(qp + 16 * s));
     }
 
     f32x16_t oacc[4];
@@ -84,42 +93,61 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillA
     float m_run = -INFINITY;      // shared by lanes l and l^32
     float l_run = 0.f;            // partial over this lane's key half
 
-    __shared__ __attribute__((aligned(16))) bf16_t sK[kPfBN * kPfLd];
-    __shared__ __attribute__((aligned(16))) bf16_t sV[kPfBN * kPfLd];
+    __shared__ __attribute__((aligned(16))) u32x4_t sK[2][kPfTileChunks];
+    __shared__ __attribute__((aligned(16))) u32x4_t sV[2][kPfTileChunks];
 
     const int q_hi = min(row0 + kPfBM, lq) - 1;          // last query row of the tile
     const int kv_end = min(lk, q_hi + off + 1);          // keys [0, kv_end) are visible to the tile
     const int ntiles = kv_end > 0 ? (kv_end + kPfBN - 1) / kPfBN : 0;
     const int wave_qmin = row0 + wave * 32;
 
-    for (int kt = 0; kt < ntiles; ++kt) {
-        __syncthreads();                                 // everyone is done with the previous tile
+    // global -> registers for key tile kt: thread t moves chunks t, t+256, t+512, t+768 of the tile
+    // (chunk c = key c/16, 16 bytes c%16); keys past the end are clamped and masked later
+    auto load_tile = [&](int kt, u32x4_t (&kr)[4], u32x4_t (&vr)[4]) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int c = tid + kPfThreads * r;          // 1024 16-byte chunks per tile
+            const int c = tid + kPfThreads * r;
             const int key = c >> 4, ch = c & 15;
-            const int kk = min(kt * kPfBN + key, lk - 1);     // rows past the end are masked below
-            uint4 kd, vd;
+            const int kk = min(kt * kPfBN + key, lk - 1);
             if (kPaged) {
                 const int32_t blk = a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + (kk >> 8)];
                 if (static_cast<uint32_t>(blk) < static_cast<uint32_t>(a.num_blocks)) {
                     const int64_t e = ((static_cast<int64_t>(blk) * kBlockSize + (kk & 255)) * a.num_kv_heads + hkv) *
                                           kHeadDim + ch * 8;
-                    kd = *reinterpret_cast<const uint4 *>(a.k_cache + e);
-                    vd = *reinterpret_cast<const uint4 *>(a.v_cache + e);
+                    kr[r] = *reinterpret_cast<const u32x4_t *>(a.k_cache + e);
+                    vr[r] = *reinterpret_cast<const u32x4_t *>(a.v_cache + e);
                 } else {
-                    kd = make_uint4(0, 0, 0, 0);
-                    vd = kd;
+                    kr[r] = u32x4_t{0u, 0u, 0u, 0u};
+                    vr[r] = u32x4_t{0u, 0u, 0u, 0u};
                 }
             } else {
                 const int64_t tok = static_cast<int64_t>(k0 + kk);
-                kd = *reinterpret_cast<const uint4 *>(a.k + tok * a.k_row_stride + hkv * kHeadDim + ch * 8);
-                vd = *reinterpret_cast<const uint4 *>(a.v + tok * a.v_row_stride + hkv * kHeadDim + ch * 8);
+                kr[r] = *reinterpret_cast<const u32x4_t *>(a.k + tok * a.k_row_stride + hkv * kHeadDim + ch * 8);
+                vr[r] = *reinterpret_cast<const u32x4_t *>(a.v + tok * a.v_row_stride + hkv * kHeadDim + ch * 8);
             }
-            *reinterpret_cast<uint4 *>(&sK[key * kPfLd + ch * 8]) = kd;
-            *reinterpret_cast<uint4 *>(&sV[key * kPfLd + ch * 8]) = vd;
         }
-        __syncthreads();
+    };
+    auto store_tile = [&](int buf, const u32x4_t (&kr)[4], const u32x4_t (&vr)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int c = tid + kPfThreads * r;
+            const int key = c >> 4, ch = c & 15;
+            sK[buf][key * 16 + (ch ^ (key & 15))] = kr[r];
+            sV[buf][key * 16 + (ch ^ (4 * (key & 3)))] = vr[r];
+        }
+    };
+
+    u32x4_t kr[4], vr[4];
+    if (ntiles > 0) {
+        load_tile(0, kr, vr);
+        store_tile(0, kr, vr);
+    }
+    __syncthreads();
+
+    for (int kt = 0; kt < ntiles; ++kt) {
+        const int buf = kt & 1;
+        const bool more = kt + 1 < ntiles;
+        if (more) load_tile(kt + 1, kr, vr);             // in flight during this tile's arithmetic
 
         // ---- S^T = K Q^T for two 32-key sub-tiles ----------------------------------------
         f32x16_t sacc[2];
@@ -129,79 +157,87 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillA
             for (int i = 0; i < 16; ++i) sacc[t2][i] = 0.f;
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
-                const uint4 kf = *reinterpret_cast<const uint4 *>(&sK[(t2 * 32 + qi) * kPfLd + 16 * s + 8 * hh]);
+                const int key = t2 * 32 + qi;
+                const u32x4_t kf = sK[buf][key * 16 + ((2 * s + hh) ^ (key & 15))];
                 sacc[t2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf), qfrag[s], sacc[t2], 0, 0, 0);
             }
         }
 
-        // ---- scale, causal mask, running softmax ------------------------------------------
-        const int key_base = kt * kPfBN + 4 * hh;
+        // ---- causal mask, running softmax (base 2; the scale is folded into the exponent) -------
+        // m_run is the running maximum of the RAW scores; p = exp2(scale*log2e * (s - m)).
         const int limit = qrow + off;                    // last key this query may see
-        const bool need_mask = (kt * kPfBN + kPfBN - 1) > (wave_qmin + off);
-        float mloc = -INFINITY;
+        if ((kt * kPfBN + kPfBN - 1) > (wave_qmin + off)) {   // only tiles that cross the diagonal
+            const int key_base = kt * kPfBN + 4 * hh;
 #pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2)
+            for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float x = sacc[t2][i] * a.scale_log2e;
-                if (need_mask) {
-                    const int key = key_base + t2 * 32 + 8 * (i >> 2) + (i & 3);
-                    if (key > limit) x = -INFINITY;
-                }
-                sacc[t2][i] = x;
-                mloc = fmaxf(mloc, x);
-            }
+                for (int i = 0; i < 16; ++i)
+                    if (key_base + t2 * 32 + 8 * (i >> 2) + (i & 3) > limit) sacc[t2][i] = -INFINITY;
+        }
+        float mloc = fmaxf(sacc[0][0], sacc[1][0]);
+#pragma unroll
+        for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(sacc[0][i], sacc[1][i]));
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
         const float m_new = fmaxf(m_run, mloc);
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;    // no key seen yet: p = 0
-        const float alpha = exp2f(m_run - m_safe);
-        m_run = m_new;
+        const float neg_ms = -m_safe * a.scale_log2e;
         float psum = 0.f;
-        uint4 pfrag[2][2];                               // [sub-tile][k-step of 16 keys]
+        u32x4_t pfrag[2][2];                             // [sub-tile][k-step of 16 keys]
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
             float p[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                p[i] = exp2f(sacc[t2][i] - m_safe);
+                p[i] = __builtin_amdgcn_exp2f(fmaf(sacc[t2][i], a.scale_log2e, neg_ms));   // exp2(-inf) = 0
                 psum += p[i];
             }
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2)
-                pfrag[t2][s2] = make_uint4(pack_bf16x2(p[8 * s2 + 0], p[8 * s2 + 1]),
-                                           pack_bf16x2(p[8 * s2 + 2], p[8 * s2 + 3]),
-                                           pack_bf16x2(p[8 * s2 + 4], p[8 * s2 + 5]),
-                                           pack_bf16x2(p[8 * s2 + 6], p[8 * s2 + 7]));
+                pfrag[t2][s2] = u32x4_t{pack_bf16x2(p[8 * s2 + 0], p[8 * s2 + 1]), pack_bf16x2(p[8 * s2 + 2], p[8 * s2 + 3]),
+                                        pack_bf16x2(p[8 * s2 + 4], p[8 * s2 + 5]), pack_bf16x2(p[8 * s2 + 6], p[8 * s2 + 7])};
         }
-        l_run = l_run * alpha + psum;
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {     // some query of the wavefront moved its maximum
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * a.scale_log2e);   // exp2(-inf) = 0 on first use
+            l_run *= alpha;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+                for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+            m_run = m_new;
+        }
+        l_run += psum;
 
         // ---- O^T += V^T P^T ----------------------------------------------------------------
-        // A operand: row = output dim (dt*32 + qi), k slot (hh, i) = key 16*s2 + 8*(i/4) + 4*hh + i%4
+        // A operand: row = output dim (dt*32 + lane%32), k slot (hh, i) = key 16*s2 + 8*(i/4) + 4*hh + i%4.
+        // Transpose read: the 16 lanes of a group fetch [4 keys][16 dims]; lane r16 supplies the address
+        // of key r16/4, dims 4*(r16%4)..+3 and receives dim r16 of the four keys.
+        {
+            const int r16 = lane & 15;
+            const int dsub = (lane >> 4) & 1;            // which 16-dim half of the 32-dim tile
+            const int kq = r16 >> 2;                     // key within the group of four
+            const int cin = dsub * 2 + ((r16 >> 1) & 1); // 16-byte chunk within the tile's 64-byte dim span
+            const char *vbase = reinterpret_cast<const char *>(&sV[buf][0]) + (r16 & 1) * 8;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-            const int dim = dt * 32 + qi;
+            for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2)
+                for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-                for (int s2 = 0; s2 < 2; ++s2) {
-                    const int kbase = t2 * 32 + 16 * s2 + 4 * hh;
-                    uint32_t w[4];
-#pragma unroll
-                    for (int pr = 0; pr < 4; ++pr) {
-                        const int ka = kbase + 8 * (pr >> 1) + 2 * (pr & 1);
-                        const uint32_t lo = sV[ka * kPfLd + dim];
-                        const uint32_t hi = sV[(ka + 1) * kPfLd + dim];
-                        w[pr] = lo | (hi << 16);
+                    for (int s2 = 0; s2 < 2; ++s2) {
+                        const int k_lo = t2 * 32 + 16 * s2 + 4 * hh + kq;     // k slots 0..3
+                        const int k_hi = k_lo + 8;                            // k slots 4..7
+                        const int c = dt * 4 + cin;
+                        const s16x4_t vlo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (lds_s16x4_ptr)(vbase + k_lo * 256 + ((c ^ (4 * (k_lo & 3))) * 16)));
+                        const s16x4_t vhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (lds_s16x4_ptr)(vbase + k_hi * 256 + ((c ^ (4 * (k_hi & 3))) * 16)));
+                        const s16x8_t both = __builtin_shufflevector(vlo, vhi, 0, 1, 2, 3, 4, 5, 6, 7);
+                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, both),
+                                                                           as_bf16x8(pfrag[t2][s2]), oacc[dt], 0, 0, 0);
                     }
-                    const uint4 vf = make_uint4(w[0], w[1], w[2], w[3]);
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf), as_bf16x8(pfrag[t2][s2]),
-                                                                       oacc[dt], 0, 0, 0);
-                }
         }
+
+        if (more) store_tile(buf ^ 1, kr, vr);           // the other buffer was last read before the previous barrier
+        __syncthreads();
     }
 
     // ---- normalise and store: register i of tile dt = dim dt*32 + 8*(i/4) + 4*hh + i%4 ----
