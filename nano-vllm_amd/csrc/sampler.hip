@@ -11,11 +11,15 @@
 // A row of 151,936 logits is far too little work for one workgroup and 64..256 rows are
 // too few workgroups for 256 CUs, so a row is cut into chunks of 2048 columns (one
 // workgroup of 256 lanes, one 16-byte load of 8 bf16 per lane):
+// With a caller-supplied noise tensor (the replayable form):
 //   pass 1  per (chunk, row): chunk max and sum exp(x - chunk max)          -> workspace
 //   pass 2  per (chunk, row): merge the row's partials into (max, sum), then
 //           best p_i / E_i and its column inside the chunk                   -> workspace
 //   pass 3  per row: best chunk, lowest column on ties                       -> int64 token
 // Pass 2 re-reads the logits (2 B/col) that pass 1 pulled through L2 / Infinity Cache.
+// With in-kernel noise there is nothing to replay against, so the draw uses the equivalent
+// Gumbel form argmax_i (x_i - log E_i), which needs no softmax: ONE pass over the logits
+// (sampler_gumbel_kernel) followed by the per-row pick -- the same exact categorical draw.
 // Algorithmic HBM bytes per row: vocab * 2 B (+ vocab * 4 B when the noise is read).
 #include "nva_common.h"
 
@@ -42,12 +46,6 @@ struct Philox {
         return c;
     }
 };
-
-// Exp(1) from 32 random bits: u in (0, 1] with 24 bits, e = -log(u) in [0, 16.64]
-__device__ __forceinline__ float exp1_from_bits(uint32_t r) {
-    const float u = (static_cast<float>(r >> 8) + 1.0f) * 5.9604644775390625e-8f;
-    return -logf(u);
-}
 
 // Loads the 8 columns [col0, col0+8) of a row as x = float(logit) / T (greedy: T = 1).
 // Columns >= vocab come back as -inf.  vec_ok: the row start is 16-byte aligned.
@@ -107,7 +105,7 @@ __device__ __forceinline__ void better(float &bs, int &bi, float s, int i) {
 
 __global__ __launch_bounds__(kSampThreads) void sampler_argmax_kernel(
     const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
-    const float *__restrict__ noise, int64_t noise_row_stride, uint64_t seed, uint64_t offset,
+    const float *__restrict__ noise, int64_t noise_row_stride,
     const float *__restrict__ part_max, const float *__restrict__ part_sum,
     float *__restrict__ part_best, int32_t *__restrict__ part_idx, int32_t vocab, int32_t nchunks) {
     const int chunk = blockIdx.x;
@@ -149,7 +147,7 @@ __global__ __launch_bounds__(kSampThreads) void sampler_argmax_kernel(
     if (greedy) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) e[i] = 1.f;
-    } else if (noise != nullptr) {
+    } else {
         const float *nrow = noise + static_cast<int64_t>(b) * noise_row_stride;
         if (((reinterpret_cast<uintptr_t>(nrow) & 15u) == 0) && col0 + 8 <= vocab) {
             const float4 a = *reinterpret_cast<const float4 *>(nrow + col0);
@@ -160,15 +158,6 @@ __global__ __launch_bounds__(kSampThreads) void sampler_argmax_kernel(
 #pragma unroll
             for (int i = 0; i < 8; ++i) e[i] = (col0 + i < vocab) ? nrow[col0 + i] : 1.f;
         }
-    } else {
-        const uint2 key = make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
-        const uint32_t o_lo = static_cast<uint32_t>(offset), o_hi = static_cast<uint32_t>(offset >> 32);
-        const uint4 r0 = Philox::draw(make_uint4(static_cast<uint32_t>(col0 >> 2), b, o_lo, o_hi), key);
-        const uint4 r1 = Philox::draw(make_uint4(static_cast<uint32_t>(col0 >> 2) + 1u, b, o_lo, o_hi), key);
-        e[0] = exp1_from_bits(r0.x); e[1] = exp1_from_bits(r0.y);
-        e[2] = exp1_from_bits(r0.z); e[3] = exp1_from_bits(r0.w);
-        e[4] = exp1_from_bits(r1.x); e[5] = exp1_from_bits(r1.y);
-        e[6] = exp1_from_bits(r1.z); e[7] = exp1_from_bits(r1.w);
     }
 
     float best = -INFINITY;
@@ -193,6 +182,68 @@ __global__ __launch_bounds__(kSampThreads) void sampler_argmax_kernel(
         const int oi = __shfl_xor(best_i, off, 64);
         better(best, best_i, os, oi);
     }
+    if (lane == 0) { sh[wave] = best; shi[wave] = best_i; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w) better(best, best_i, sh[w], shi[w]);
+        part_best[static_cast<int64_t>(b) * nchunks + chunk] = best;
+        part_idx[static_cast<int64_t>(b) * nchunks + chunk] = best_i;
+    }
+}
+
+// In-kernel noise: score_i = logit_i * log2(e)/T - log2(-log2(u_i)), u_i uniform in (0,1) from Philox.
+// (E_i = -ln(u_i); log2(E_i) = log2(-log2(u_i)) + const, and constants do not move the argmax.)
+// Greedy rows (T == 0) use score_i = logit_i.
+__global__ __launch_bounds__(kSampThreads) void sampler_gumbel_kernel(
+    const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
+    uint64_t seed, uint64_t offset, float *__restrict__ part_best, int32_t *__restrict__ part_idx,
+    int32_t vocab, int32_t nchunks) {
+    const int chunk = blockIdx.x;
+    const int b = blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const bf16_t *row = logits + static_cast<int64_t>(b) * row_stride;
+    const bool vec_ok = ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
+    const float t_in = temperatures[b];
+    const bool greedy = (t_in == 0.f);
+    const float k = greedy ? 1.f : 1.4426950408889634f / t_in;
+    const int col0 = chunk * kSampChunk + threadIdx.x * 8;
+    float x[8];
+    if (vec_ok && col0 + 8 <= vocab) {
+        unpack8(*reinterpret_cast<const uint4 *>(row + col0), x);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = (col0 + i < vocab) ? bf16_to_f32(row[col0 + i]) : -INFINITY;
+    }
+    float g[8];
+    if (greedy) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) g[i] = 0.f;
+    } else {
+        const uint2 key = make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+        const uint32_t o_lo = static_cast<uint32_t>(offset), o_hi = static_cast<uint32_t>(offset >> 32);
+        const uint4 r0 = Philox::draw(make_uint4(static_cast<uint32_t>(col0 >> 2), b, o_lo, o_hi), key);
+        const uint4 r1 = Philox::draw(make_uint4(static_cast<uint32_t>(col0 >> 2) + 1u, b, o_lo, o_hi), key);
+        const uint32_t r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            // u in (0, 1): 23 random bits plus one half, so that neither log below sees 0 or 1
+            const float u = (static_cast<float>(r[i] >> 9) + 0.5f) * 1.1920928955078125e-7f;
+            g[i] = __builtin_amdgcn_logf(-__builtin_amdgcn_logf(u));      // log2(-log2 u)
+        }
+    }
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        if (col0 + i < vocab) better(best, best_i, fmaf(x[i], k, -g[i]), col0 + i);
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float os = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(best_i, off, 64);
+        better(best, best_i, os, oi);
+    }
+    __shared__ float sh[4];
+    __shared__ int shi[4];
     if (lane == 0) { sh[wave] = best; shi[wave] = best_i; }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -248,11 +299,19 @@ extern "C" int nva_sample(const void *logits, int64_t logits_row_stride, const f
     int32_t *part_idx = reinterpret_cast<int32_t *>(part_best + n);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bf16_t *lg = static_cast<const bf16_t *>(logits);
+    if (noise == nullptr) {
+        hipLaunchKernelGGL(sampler_gumbel_kernel, dim3(nchunks, batch), dim3(kSampThreads), 0, s, lg,
+                           logits_row_stride, temperatures, seed, offset, part_best, part_idx, vocab, nchunks);
+        if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
+        hipLaunchKernelGGL(sampler_pick_kernel, dim3(batch), dim3(kWave), 0, s, part_best, part_idx, out_tokens,
+                           nchunks);
+        return launch_status();
+    }
     hipLaunchKernelGGL(sampler_partials_kernel, dim3(nchunks, batch), dim3(kSampThreads), 0, s, lg,
                        logits_row_stride, temperatures, part_max, part_sum, vocab, nchunks);
     if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
     hipLaunchKernelGGL(sampler_argmax_kernel, dim3(nchunks, batch), dim3(kSampThreads), 0, s, lg,
-                       logits_row_stride, temperatures, noise, noise_row_stride, seed, offset, part_max,
+                       logits_row_stride, temperatures, noise, noise_row_stride, part_max,
                        part_sum, part_best, part_idx, vocab, nchunks);
     if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
     hipLaunchKernelGGL(sampler_pick_kernel, dim3(batch), dim3(kWave), 0, s, part_best, part_idx, out_tokens,

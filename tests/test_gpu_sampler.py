@@ -91,3 +91,26 @@ def test_sampler_philox_mode_is_categorical_and_reproducible(dev):
     s = Sampler(seed=3)
     x, y = s(logits, temps).cpu(), s(logits, temps).cpu()
     assert x.shape == (n,) and not torch.equal(x, y)
+
+
+def test_sampler_philox_mode_large_vocab_and_greedy(dev):
+    """In-kernel noise on a wide, flat vocabulary: bucketed chi-square against the softmax, a
+    dominant logit always wins, and temperature-0 rows are plain argmax."""
+    v, n, t = 4096, 50000, 1.0
+    g = torch.Generator().manual_seed(3)
+    row = (torch.randn(v, generator=g) * 0.5).to(torch.bfloat16)
+    logits = row.expand(n, v).contiguous().to(dev)
+    tok = sample(logits, torch.full((n,), t, device=dev), None, seed=5, offset=9).cpu()
+    p = torch.softmax(row.double() / t, -1)
+    buckets = 64
+    freq = torch.bincount(tok // (v // buckets), minlength=buckets).double()
+    pb = p.view(buckets, -1).sum(-1)
+    chi2 = float(((freq - n * pb) ** 2 / (n * pb)).sum())
+    assert chi2 < 130.0, chi2                     # 63 dof: P(chi2 > 130) ~ 1e-6
+    peaked = torch.zeros(8, 151936, dtype=torch.bfloat16)
+    peaked[torch.arange(8), torch.arange(8) * 18000 + 7] = 60.0
+    out = sample(peaked.to(dev), torch.full((8,), 0.6, device=dev), None, seed=1, offset=1).cpu()
+    assert out.tolist() == [i * 18000 + 7 for i in range(8)]
+    case = synthetic.sampler_case(seed=8, batch=16, vocab=151936)
+    out = sample(case.logits.to(dev), torch.zeros(16, device=dev), None, seed=2, offset=3).cpu()
+    assert torch.equal(out, case.logits.float().argmax(-1))
