@@ -167,12 +167,12 @@ int nva_rms_norm(const void *x, int64_t x_row_stride,
  * qkv: bf16 [n_tokens, (num_heads + 2*num_kv_heads) * head_dim], row stride in elements
  * (q heads, then k heads, then v heads; v is left untouched).  positions: int64 [n_tokens].
  * q_weight / k_weight: bf16 [head_dim].  rope_cache: fp32 [max_position, head_dim], cos in
- * the first half of a row, sin in the second.  q_out: bf16 [n_tokens, num_heads, head_dim],
+ * the first half of a row, sin in the second; positions are clamped to [0, max_position).  q_out: bf16 [n_tokens, num_heads, head_dim],
  * k_out: bf16 [n_tokens, num_kv_heads, head_dim], both dense.  head_dim must be 128.
  */
 int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const int64_t *positions,
                      const void *q_weight, const void *k_weight, const float *rope_cache,
-                     void *q_out, void *k_out,
+                     int32_t max_position, void *q_out, void *k_out,
                      int32_t n_tokens, int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
                      float eps, void *stream);
 

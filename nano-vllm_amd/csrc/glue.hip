@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(
     const bf16_t *__restrict__ qkv, int64_t row_stride, const int64_t *__restrict__ positions,
     const bf16_t *__restrict__ q_weight, const bf16_t *__restrict__ k_weight,
     const float *__restrict__ rope_cache, bf16_t *__restrict__ q_out, bf16_t *__restrict__ k_out,
-    int64_t n_rows, int32_t hq, int32_t hkv, float eps) {
+    int64_t n_rows, int32_t hq, int32_t hkv, int32_t max_position, float eps) {
     const int lane = threadIdx.x & 63;
     const int64_t r = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (r >= n_rows) return;
@@ -97,7 +97,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(
     const float inv = rsqrtf(ss * (1.0f / kHeadDim) + eps);
     const float y1 = round_bf16(round_bf16(x1 * inv) * bf16_to_f32(w[lane]));
     const float y2 = round_bf16(round_bf16(x2 * inv) * bf16_to_f32(w[lane + 64]));
-    const float *cs = rope_cache + positions[tok] * kHeadDim;
+    // positions outside the table are clamped instead of read out of bounds
+    const int64_t pos = min(max(positions[tok], static_cast<int64_t>(0)), static_cast<int64_t>(max_position) - 1);
+    const float *cs = rope_cache + pos * kHeadDim;
     const float c = cs[lane], s = cs[lane + 64];
     bf16_t *dst = is_q ? q_out + (tok * hq + head) * kHeadDim : k_out + (tok * hkv + (head - hq)) * kHeadDim;
     dst[lane] = f32_to_bf16(y1 * c - y2 * s);
@@ -149,10 +151,10 @@ extern "C" int nva_rms_norm(const void *x, int64_t x_row_stride, const void *res
 
 extern "C" int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const int64_t *positions,
                                 const void *q_weight, const void *k_weight, const float *rope_cache,
-                                void *q_out, void *k_out, int32_t n_tokens, int32_t num_heads,
+                                int32_t max_position, void *q_out, void *k_out, int32_t n_tokens, int32_t num_heads,
                                 int32_t num_kv_heads, int32_t head_dim, float eps, void *stream) {
     using namespace nva;
-    if (n_tokens < 0 || num_heads <= 0 || num_kv_heads <= 0) return NVA_ERR_BAD_SHAPE;
+    if (n_tokens < 0 || num_heads <= 0 || num_kv_heads <= 0 || max_position <= 0) return NVA_ERR_BAD_SHAPE;
     if (head_dim != kHeadDim) return NVA_ERR_UNSUPPORTED_GEOMETRY;
     if (n_tokens == 0) return NVA_OK;
     if (!qkv || !positions || !q_weight || !k_weight || !rope_cache || !q_out || !k_out) return NVA_ERR_NULL_POINTER;
@@ -162,7 +164,7 @@ extern "C" int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const i
     hipLaunchKernelGGL(qk_norm_rope_kernel, dim3(static_cast<uint32_t>((n_rows + 3) / 4)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const bf16_t *>(qkv), qkv_row_stride, positions,
                        static_cast<const bf16_t *>(q_weight), static_cast<const bf16_t *>(k_weight), rope_cache,
-                       static_cast<bf16_t *>(q_out), static_cast<bf16_t *>(k_out), n_rows, num_heads, num_kv_heads, eps);
+                       static_cast<bf16_t *>(q_out), static_cast<bf16_t *>(k_out), n_rows, num_heads, num_kv_heads, max_position, eps);
     return launch_status();
 }
 

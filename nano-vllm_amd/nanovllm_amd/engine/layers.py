@@ -64,7 +64,7 @@ def qk_norm_rope(qkv: torch.Tensor, positions: torch.Tensor, q_weight: torch.Ten
     q = torch.empty((n, num_heads, head_dim), dtype=_BF16, device=qkv.device)
     k = torch.empty((n, num_kv_heads, head_dim), dtype=_BF16, device=qkv.device)
     rc = _lib.load().nva_qk_norm_rope(qkv.data_ptr(), qkv.stride(0), positions.data_ptr(), q_weight.data_ptr(),
-                                      k_weight.data_ptr(), rope_cache.data_ptr(), q.data_ptr(), k.data_ptr(),
+                                      k_weight.data_ptr(), rope_cache.data_ptr(), rope_cache.shape[0], q.data_ptr(), k.data_ptr(),
                                       n, num_heads, num_kv_heads, head_dim, float(eps), _stream())
     _lib.check(rc, "nva_qk_norm_rope")
     v = qkv[:, (num_heads + num_kv_heads) * head_dim:].view(n, num_kv_heads, head_dim)

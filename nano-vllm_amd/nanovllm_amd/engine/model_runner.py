@@ -13,7 +13,7 @@ from typing import List, Optional
 import numpy as np
 import torch
 
-from ..context import get_context, reset_context, set_context
+from ..context import reset_context, set_context
 from ..sampler import Sampler
 from .config import EngineConfig
 from .model import Qwen3ForCausalLM
@@ -159,29 +159,60 @@ class ModelRunner:
                                torch.float32)
 
     # ---- execution -----------------------------------------------------------------------------
+    def _init_decode_staging(self, max_bs: int) -> None:
+        """One pinned host buffer and one device buffer holding every per-step decode input; the
+        graph's static tensors are typed views into the device buffer, so a decode step needs a
+        single host-to-device copy (the reference issues one copy per tensor plus one device copy
+        per graph variable, nanovllm/engine/model_runner.py:162-179,197-203)."""
+        fields = [("input_ids", np.int64, (max_bs,)), ("positions", np.int64, (max_bs,)),
+                  ("slot_mapping", np.int32, (max_bs,)), ("context_lens", np.int32, (max_bs,)),
+                  ("temperatures", np.float32, (max_bs,)), ("block_tables", np.int32, (max_bs, self.max_table_width))]
+        offsets, total = {}, 0
+        for name, dt, shape in fields:
+            nbytes = int(np.prod(shape)) * np.dtype(dt).itemsize
+            offsets[name] = (total, nbytes, dt, shape)
+            total += (nbytes + 255) // 256 * 256
+        # zero-filled: rows past the batch are replayed too (bucket padding) and must hold valid ids / positions
+        self._stage_host = torch.zeros(total, dtype=torch.uint8).pin_memory()
+        self._stage_dev = torch.zeros(total, dtype=torch.uint8, device=self.device)
+        host_np = self._stage_host.numpy()
+        tdt = {np.int64: torch.int64, np.int32: torch.int32, np.float32: torch.float32}
+        self._stage_np, self.graph_vars = {}, {}
+        for name, (off, nbytes, dt, shape) in offsets.items():
+            self._stage_np[name] = host_np[off: off + nbytes].view(dt).reshape(shape)
+            self.graph_vars[name] = self._stage_dev[off: off + nbytes].view(tdt[dt]).view(shape)
+
+    def _run_decode_graph(self, seqs: List[Sequence]) -> torch.Tensor:
+        """Fill the staging buffer, copy it once, replay the bucket's graph; returns logits."""
+        bs = len(seqs)
+        bucket = next(x for x in self.graph_bs if x >= bs)
+        h = build_decode_inputs(seqs, self.block_size)
+        st = self._stage_np
+        st["input_ids"][:bs] = h["input_ids"]
+        st["positions"][:bs] = h["positions"]
+        st["slot_mapping"][:bs] = h["slot_mapping"]
+        st["slot_mapping"][bs:bucket] = -1                        # padded rows store nothing ...
+        st["context_lens"][:bs] = h["context_lens"]
+        st["context_lens"][bs:bucket] = 0                         # ... and attend over nothing
+        st["temperatures"][:bs] = np.fromiter((s.temperature for s in seqs), dtype=np.float32, count=bs)
+        st["block_tables"][:bs, : h["block_tables"].shape[1]] = h["block_tables"]   # stale columns stay: never read
+        self._stage_dev.copy_(self._stage_host, non_blocking=True)
+        self.graphs[bucket].replay()
+        return self.model.compute_logits(self.graph_vars["outputs"][:bs])
+
     @torch.inference_mode()
     def run_model(self, input_ids: torch.Tensor, positions: torch.Tensor, is_prefill: bool) -> torch.Tensor:
-        bs = input_ids.size(0)
-        if is_prefill or self.enforce_eager or not self.graph_bs or bs > self.graph_bs[-1]:
-            return self.model.compute_logits(self.model(input_ids, positions))
-        ctx = get_context()
-        bucket = next(x for x in self.graph_bs if x >= bs)
-        gv = self.graph_vars
-        gv["input_ids"][:bs] = input_ids
-        gv["positions"][:bs] = positions
-        gv["slot_mapping"].fill_(-1)                              # padded rows store nothing ...
-        gv["slot_mapping"][:bs] = ctx.slot_mapping
-        gv["context_lens"].zero_()                                # ... and attend over nothing
-        gv["context_lens"][:bs] = ctx.context_lens
-        gv["block_tables"][:bs, : ctx.block_tables.size(1)] = ctx.block_tables   # stale columns stay: never read
-        self.graphs[bucket].replay()
-        return self.model.compute_logits(gv["outputs"][:bs])
+        return self.model.compute_logits(self.model(input_ids, positions))
 
     def run(self, seqs: List[Sequence], is_prefill: bool) -> List[int]:
         with torch.inference_mode():
-            input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
-            temperatures = self.prepare_sample(seqs)
-            logits = self.run_model(input_ids, positions, is_prefill)
+            if not is_prefill and self.graph_bs and len(seqs) <= self.graph_bs[-1]:
+                logits = self._run_decode_graph(seqs)
+                temperatures = self.graph_vars["temperatures"][: len(seqs)]
+            else:
+                input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
+                temperatures = self.prepare_sample(seqs)
+                logits = self.run_model(input_ids, positions, is_prefill)
             tokens = self.sampler(logits, temperatures).tolist()   # the one device->host sync per step
         reset_context()
         return tokens
@@ -190,13 +221,11 @@ class ModelRunner:
     def capture_graphs(self) -> None:
         cfg = self.config
         max_bs = min(cfg.max_num_seqs, 512)
-        dev = self.device
-        input_ids = torch.zeros(max_bs, dtype=torch.int64, device=dev)
-        positions = torch.zeros(max_bs, dtype=torch.int64, device=dev)
-        slot_mapping = torch.zeros(max_bs, dtype=torch.int32, device=dev)
-        context_lens = torch.zeros(max_bs, dtype=torch.int32, device=dev)
-        block_tables = torch.zeros(max_bs, self.max_table_width, dtype=torch.int32, device=dev)
-        outputs = torch.zeros(max_bs, self.cfg.hidden_size, dtype=torch.bfloat16, device=dev)
+        self._init_decode_staging(max_bs)
+        gv = self.graph_vars
+        input_ids, positions, slot_mapping = gv["input_ids"], gv["positions"], gv["slot_mapping"]
+        context_lens, block_tables = gv["context_lens"], gv["block_tables"]
+        outputs = torch.zeros(max_bs, self.cfg.hidden_size, dtype=torch.bfloat16, device=self.device)
         self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))
         pool = None
         for bs in reversed(self.graph_bs):
@@ -212,5 +241,4 @@ class ModelRunner:
             torch.cuda.synchronize()
             reset_context()
         self.graph_pool = pool
-        self.graph_vars = dict(input_ids=input_ids, positions=positions, slot_mapping=slot_mapping,
-                               context_lens=context_lens, block_tables=block_tables, outputs=outputs)
+        self.graph_vars["outputs"] = outputs
