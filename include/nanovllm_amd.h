@@ -146,7 +146,9 @@ int nva_sample(const void *logits, int64_t logits_row_stride,
 
 /*
  * ---- steps either side of the hot path (the callers' element-wise glue) ----------------
- *
+ */
+
+/*
  * RMSNorm, optionally fused with the residual add.  Replaces RMSNorm.rms_forward /
  * add_rms_forward (nanovllm/layers/layernorm.py:16-40).
  *   residual == NULL: out = bf16(x * rsqrt(mean(x^2) + eps)) * weight
@@ -161,18 +163,26 @@ int nva_rms_norm(const void *x, int64_t x_row_stride,
                  int32_t rows, int32_t hidden, float eps, void *stream);
 
 /*
- * Per-head RMSNorm of q and k followed by the neox rotary embedding.  Replaces the q_norm /
- * k_norm / rotary_emb sequence of Qwen3Attention.forward (nanovllm/models/qwen3.py:76-79;
- * nanovllm/layers/rotary_embedding.py:6-48).
+ * Per-head RMSNorm of q and k followed by the neox rotary embedding, optionally fused with the
+ * KV-cache scatter.  Replaces the q_norm / k_norm / rotary_emb sequence of
+ * Qwen3Attention.forward (nanovllm/models/qwen3.py:76-79; nanovllm/layers/rotary_embedding.py:6-48)
+ * and, when a cache is given, the store_kvcache call of Attention.forward
+ * (nanovllm/layers/attention.py:62-63) for the same rows.
  * qkv: bf16 [n_tokens, (num_heads + 2*num_kv_heads) * head_dim], row stride in elements
- * (q heads, then k heads, then v heads; v is left untouched).  positions: int64 [n_tokens].
+ * (q heads, then k heads, then v heads).  positions: int64 [n_tokens].
  * q_weight / k_weight: bf16 [head_dim].  rope_cache: fp32 [max_position, head_dim], cos in
- * the first half of a row, sin in the second; positions are clamped to [0, max_position).  q_out: bf16 [n_tokens, num_heads, head_dim],
- * k_out: bf16 [n_tokens, num_kv_heads, head_dim], both dense.  head_dim must be 128.
+ * the first half of a row, sin in the second; positions are clamped to [0, max_position).
+ * q_out: bf16 [n_tokens, num_heads, head_dim], k_out: bf16 [n_tokens, num_kv_heads, head_dim],
+ * both dense.  head_dim must be 128.
+ * k_cache / v_cache / slot_mapping: all NULL (no scatter), or the flat caches
+ * [num_slots, num_kv_heads * head_dim] and int32 [n_tokens] slots: the rotated key row and the
+ * (unchanged) value row of token i are also written to cache row slot_mapping[i], bit-identical
+ * to what nva_store_kvcache would write from k_out and the v view; -1 / out-of-range skips.
  */
 int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const int64_t *positions,
                      const void *q_weight, const void *k_weight, const float *rope_cache,
                      int32_t max_position, void *q_out, void *k_out,
+                     void *k_cache, void *v_cache, const int32_t *slot_mapping, int64_t num_slots,
                      int32_t n_tokens, int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
                      float eps, void *stream);
 

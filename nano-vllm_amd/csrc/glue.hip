@@ -76,20 +76,35 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
 
 // One wavefront per (token, head) row of 128 elements; lane l holds elements l and l + 64,
 // which are exactly the pair the neox rotation mixes.  Heads [0, hq) are queries, [hq, hq+hkv)
-// keys; values are not touched (the attention layer reads them in place).
+// keys.  With a cache (k_cache != nullptr) the rotated key row is also written to its cache slot
+// and rows [hq+hkv, hq+2*hkv) copy the value heads to theirs -- the KV scatter fused into the
+// step that produces k (slot -1 or out of range skips the row); without a cache the value rows
+// are not visited at all.
 __global__ __launch_bounds__(256) void qk_norm_rope_kernel(
     const bf16_t *__restrict__ qkv, int64_t row_stride, const int64_t *__restrict__ positions,
     const bf16_t *__restrict__ q_weight, const bf16_t *__restrict__ k_weight,
     const float *__restrict__ rope_cache, bf16_t *__restrict__ q_out, bf16_t *__restrict__ k_out,
-    int64_t n_rows, int32_t hq, int32_t hkv, int32_t max_position, float eps) {
+    bf16_t *__restrict__ k_cache, bf16_t *__restrict__ v_cache, const int32_t *__restrict__ slot_mapping,
+    int64_t num_slots, int64_t n_rows, int32_t hq, int32_t hkv, int32_t heads, int32_t max_position, float eps) {
     const int lane = threadIdx.x & 63;
     const int64_t r = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (r >= n_rows) return;
-    const int heads = hq + hkv;
     const int64_t tok = r / heads;
     const int head = static_cast<int>(r % heads);
+    const bf16_t *src = qkv + tok * row_stride + head * kHeadDim;     // q, k and v heads are adjacent
+    int64_t slot = -1;
+    if (k_cache != nullptr && head >= hq) {
+        slot = slot_mapping[tok];
+        if (slot >= num_slots) slot = -1;
+    }
+    if (head >= hq + hkv) {                                            // value head: cache write only
+        if (slot >= 0) {
+            bf16_t *dst = v_cache + (slot * hkv + (head - hq - hkv)) * kHeadDim;
+            reinterpret_cast<uint32_t *>(dst)[lane] = reinterpret_cast<const uint32_t *>(src)[lane];
+        }
+        return;
+    }
     const bool is_q = head < hq;
-    const bf16_t *src = qkv + tok * row_stride + head * kHeadDim;     // q heads then k heads are adjacent
     const bf16_t *w = is_q ? q_weight : k_weight;
     const float x1 = bf16_to_f32(src[lane]);
     const float x2 = bf16_to_f32(src[lane + 64]);
@@ -101,9 +116,16 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(
     const int64_t pos = min(max(positions[tok], static_cast<int64_t>(0)), static_cast<int64_t>(max_position) - 1);
     const float *cs = rope_cache + pos * kHeadDim;
     const float c = cs[lane], s = cs[lane + 64];
+    const bf16_t o1 = f32_to_bf16(y1 * c - y2 * s);
+    const bf16_t o2 = f32_to_bf16(y2 * c + y1 * s);
     bf16_t *dst = is_q ? q_out + (tok * hq + head) * kHeadDim : k_out + (tok * hkv + (head - hq)) * kHeadDim;
-    dst[lane] = f32_to_bf16(y1 * c - y2 * s);
-    dst[lane + 64] = f32_to_bf16(y2 * c + y1 * s);
+    dst[lane] = o1;
+    dst[lane + 64] = o2;
+    if (slot >= 0) {
+        bf16_t *cd = k_cache + (slot * hkv + (head - hq)) * kHeadDim;
+        cd[lane] = o1;
+        cd[lane + 64] = o2;
+    }
 }
 
 // out[r, i] = bf16(silu(x[r, i])) * x[r, inter + i], 8 elements per lane
@@ -151,20 +173,31 @@ extern "C" int nva_rms_norm(const void *x, int64_t x_row_stride, const void *res
 
 extern "C" int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const int64_t *positions,
                                 const void *q_weight, const void *k_weight, const float *rope_cache,
-                                int32_t max_position, void *q_out, void *k_out, int32_t n_tokens, int32_t num_heads,
-                                int32_t num_kv_heads, int32_t head_dim, float eps, void *stream) {
+                                int32_t max_position, void *q_out, void *k_out, void *k_cache, void *v_cache,
+                                const int32_t *slot_mapping, int64_t num_slots, int32_t n_tokens,
+                                int32_t num_heads, int32_t num_kv_heads, int32_t head_dim, float eps,
+                                void *stream) {
     using namespace nva;
-    if (n_tokens < 0 || num_heads <= 0 || num_kv_heads <= 0 || max_position <= 0) return NVA_ERR_BAD_SHAPE;
+    if (n_tokens < 0 || num_heads <= 0 || num_kv_heads <= 0 || max_position <= 0 || num_slots < 0)
+        return NVA_ERR_BAD_SHAPE;
     if (head_dim != kHeadDim) return NVA_ERR_UNSUPPORTED_GEOMETRY;
     if (n_tokens == 0) return NVA_OK;
     if (!qkv || !positions || !q_weight || !k_weight || !rope_cache || !q_out || !k_out) return NVA_ERR_NULL_POINTER;
-    if (qkv_row_stride < static_cast<int64_t>(num_heads + 2 * num_kv_heads) * head_dim) return NVA_ERR_BAD_STRIDE;
-    const int64_t n_rows = static_cast<int64_t>(n_tokens) * (num_heads + num_kv_heads);
+    const bool store = k_cache != nullptr || v_cache != nullptr || slot_mapping != nullptr;
+    if (store && (!k_cache || !v_cache || !slot_mapping)) return NVA_ERR_NULL_POINTER;
+    if (qkv_row_stride < static_cast<int64_t>(num_heads + 2 * num_kv_heads) * head_dim || qkv_row_stride % 2 != 0)
+        return NVA_ERR_BAD_STRIDE;
+    if ((reinterpret_cast<uintptr_t>(qkv) & 3u) || (store && ((reinterpret_cast<uintptr_t>(v_cache) & 3u))))
+        return NVA_ERR_MISALIGNED;
+    const int32_t heads = num_heads + (store ? 2 : 1) * num_kv_heads;   // value rows only when they are stored
+    const int64_t n_rows = static_cast<int64_t>(n_tokens) * heads;
     if ((n_rows + 3) / 4 > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;
     hipLaunchKernelGGL(qk_norm_rope_kernel, dim3(static_cast<uint32_t>((n_rows + 3) / 4)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const bf16_t *>(qkv), qkv_row_stride, positions,
                        static_cast<const bf16_t *>(q_weight), static_cast<const bf16_t *>(k_weight), rope_cache,
-                       static_cast<bf16_t *>(q_out), static_cast<bf16_t *>(k_out), n_rows, num_heads, num_kv_heads, max_position, eps);
+                       static_cast<bf16_t *>(q_out), static_cast<bf16_t *>(k_out), static_cast<bf16_t *>(k_cache),
+                       static_cast<bf16_t *>(v_cache), slot_mapping, num_slots, n_rows, num_heads, num_kv_heads,
+                       heads, max_position, eps);
     return launch_status();
 }
 

@@ -177,11 +177,14 @@ class Attention(nn.Module):
         self.num_kv_heads = num_kv_heads
         self.k_cache = self.v_cache = torch.tensor([])
 
-    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kv_stored: bool = False) -> torch.Tensor:
+        """``kv_stored=True`` says the caller already wrote this step's K/V rows to the cache
+        (the fused norm + rope + scatter kernel does); the default keeps the reference's
+        behaviour of scattering here."""
         ctx = get_context()
         k_cache, v_cache = self.k_cache, self.v_cache
         have_cache = k_cache.numel() > 0 and v_cache.numel() > 0
-        if have_cache:
+        if have_cache and not kv_stored:
             store_kvcache(k, v, k_cache, v_cache, ctx.slot_mapping)
         if ctx.is_prefill:
             paged = ctx.block_tables is not None       # some sequence reads cached prefix blocks

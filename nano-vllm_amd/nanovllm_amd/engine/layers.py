@@ -50,11 +50,16 @@ def build_rope_cache(head_dim: int, max_position: int, base: float, device) -> t
 
 
 def qk_norm_rope(qkv: torch.Tensor, positions: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor,
-                 rope_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, eps: float):
-    """Per-head RMSNorm of q and k, then the rotary embedding.
+                 rope_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, eps: float,
+                 kv_store=None):
+    """Per-head RMSNorm of q and k, then the rotary embedding; optionally also the KV scatter.
 
     Returns ``(q, k, v)`` with q, k fresh contiguous ``[N, H, Dh]`` tensors and v a strided
     view into ``qkv`` -- the layouts nanovllm/models/qwen3.py:74-79 hands to the attention layer.
+    ``kv_store=(k_cache, v_cache, slot_mapping)`` additionally writes the rotated key rows and
+    the value rows to their cache slots in the same kernel (what ``store_kvcache`` would do
+    next, nanovllm/layers/attention.py:62-63); the attention layer is then called with
+    ``kv_stored=True``.
     """
     n = qkv.shape[0]
     assert qkv.dim() == 2 and qkv.dtype == _BF16 and qkv.stride(1) == 1 and qkv.is_cuda
@@ -63,8 +68,17 @@ def qk_norm_rope(qkv: torch.Tensor, positions: torch.Tensor, q_weight: torch.Ten
     assert rope_cache.dtype == torch.float32 and rope_cache.is_contiguous() and rope_cache.shape[1] == head_dim
     q = torch.empty((n, num_heads, head_dim), dtype=_BF16, device=qkv.device)
     k = torch.empty((n, num_kv_heads, head_dim), dtype=_BF16, device=qkv.device)
+    kc = vc = sm = None
+    num_slots = 0
+    if kv_store is not None:
+        k_cache, v_cache, slot_mapping = kv_store
+        d = num_kv_heads * head_dim
+        assert k_cache.dtype == _BF16 and v_cache.dtype == _BF16 and k_cache.stride(1) == d and v_cache.stride(1) == d
+        assert slot_mapping.dtype == torch.int32 and slot_mapping.numel() == n and slot_mapping.is_contiguous()
+        kc, vc, sm, num_slots = k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(), k_cache.numel() // d
     rc = _lib.load().nva_qk_norm_rope(qkv.data_ptr(), qkv.stride(0), positions.data_ptr(), q_weight.data_ptr(),
-                                      k_weight.data_ptr(), rope_cache.data_ptr(), rope_cache.shape[0], q.data_ptr(), k.data_ptr(),
+                                      k_weight.data_ptr(), rope_cache.data_ptr(), rope_cache.shape[0],
+                                      q.data_ptr(), k.data_ptr(), kc, vc, sm, num_slots,
                                       n, num_heads, num_kv_heads, head_dim, float(eps), _stream())
     _lib.check(rc, "nva_qk_norm_rope")
     v = qkv[:, (num_heads + num_kv_heads) * head_dim:].view(n, num_kv_heads, head_dim)

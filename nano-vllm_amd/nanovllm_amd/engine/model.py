@@ -41,9 +41,13 @@ class DecoderLayer(nn.Module):
         else:
             hidden, residual = layers.add_rms_norm(hidden, residual, self.input_layernorm, self.eps)
         qkv = F.linear(hidden, self.qkv_proj)
+        attn = self.attn
+        fused_store = attn.k_cache.numel() > 0                 # no cache yet during the warm-up pass
         q, k, v = layers.qk_norm_rope(qkv, positions, self.q_norm, self.k_norm, self.rope_cache,
-                                      self.num_heads, self.num_kv_heads, self.head_dim, self.eps)
-        o = self.attn(q, k, v)
+                                      self.num_heads, self.num_kv_heads, self.head_dim, self.eps,
+                                      kv_store=(attn.k_cache, attn.v_cache, get_context().slot_mapping)
+                                      if fused_store else None)
+        o = attn(q, k, v, kv_stored=fused_store)
         hidden = F.linear(o.flatten(1, -1), self.o_proj)
         hidden, residual = layers.add_rms_norm(hidden, residual, self.post_attention_layernorm, self.eps)
         hidden = F.linear(layers.silu_and_mul(F.linear(hidden, self.gate_up_proj)), self.down_proj)
@@ -68,10 +72,19 @@ class Qwen3ForCausalLM(nn.Module):
                     p.normal_(0.0, 0.02, generator=gen)
 
     def forward(self, input_ids: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
-        hidden = F.embedding(input_ids, self.embed_tokens)
-        residual = None
-        for layer in self.layers:
+        hidden, residual = self.forward_layers(input_ids, positions, None, None, 0, len(self.layers))
+        return self.finish(hidden, residual)
+
+    def forward_layers(self, input_ids, positions, hidden, residual, first: int, last: int):
+        """Layers ``[first, last)``; the embedding lookup is part of the slice that starts at 0.
+        Lets the runner capture the stack as several consecutive graphs."""
+        if first == 0:
+            hidden, residual = F.embedding(input_ids, self.embed_tokens), None
+        for layer in self.layers[first:last]:
             hidden, residual = layer(positions, hidden, residual)
+        return hidden, residual
+
+    def finish(self, hidden, residual) -> torch.Tensor:
         hidden, _ = layers.add_rms_norm(hidden, residual, self.norm, self.cfg.rms_norm_eps)
         return hidden
 

@@ -92,6 +92,8 @@ class ModelRunner:
         self.max_table_width = -(-config.max_model_len // self.block_size)
         self.graphs = {}
         self.graph_bs: List[int] = []
+        self.graph_segments = 4                          # consecutive graphs per decode step (see capture_graphs)
+        self._graph_keepalive = []
         with torch.inference_mode():
             self.warmup_model()
             self.allocate_kv_cache()
@@ -197,7 +199,8 @@ class ModelRunner:
         st["temperatures"][:bs] = np.fromiter((s.temperature for s in seqs), dtype=np.float32, count=bs)
         st["block_tables"][:bs, : h["block_tables"].shape[1]] = h["block_tables"]   # stale columns stay: never read
         self._stage_dev.copy_(self._stage_host, non_blocking=True)
-        self.graphs[bucket].replay()
+        for graph in self.graphs[bucket]:                         # later segments are enqueued while the first runs
+            graph.replay()
         return self.model.compute_logits(self.graph_vars["outputs"][:bs])
 
     @torch.inference_mode()
@@ -227,17 +230,30 @@ class ModelRunner:
         context_lens, block_tables = gv["context_lens"], gv["block_tables"]
         outputs = torch.zeros(max_bs, self.cfg.hidden_size, dtype=torch.bfloat16, device=self.device)
         self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))
+        # The layer stack of a bucket is captured as several consecutive graphs instead of one:
+        # launching a graph costs the host about a microsecond per node before the first kernel
+        # starts, and with segments only the first segment's launch is exposed -- the others are
+        # enqueued while the GPU already runs.
+        n_layers = len(self.model.layers)
+        cuts = sorted({round(i * n_layers / self.graph_segments) for i in range(self.graph_segments + 1)})
         pool = None
         for bs in reversed(self.graph_bs):
-            graph = torch.cuda.CUDAGraph()
             set_context(False, slot_mapping=slot_mapping[:bs], context_lens=context_lens[:bs],
                         block_tables=block_tables[:bs])
             outputs[:bs] = self.model(input_ids[:bs], positions[:bs])        # eager warm-up (sizes workspaces)
-            with torch.cuda.graph(graph, pool):
-                outputs[:bs] = self.model(input_ids[:bs], positions[:bs])
-            if pool is None:
-                pool = graph.pool()
-            self.graphs[bs] = graph
+            segments, hidden, residual = [], None, None
+            for first, last in zip(cuts[:-1], cuts[1:]):
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, pool):
+                    hidden, residual = self.model.forward_layers(input_ids[:bs], positions[:bs], hidden, residual,
+                                                                 first, last)
+                    if last == n_layers:
+                        outputs[:bs] = self.model.finish(hidden, residual)
+                if pool is None:
+                    pool = graph.pool()
+                segments.append((graph, hidden, residual))      # keep the boundary activations alive
+            self.graphs[bs] = [g for g, _, _ in segments]
+            self._graph_keepalive.append(segments)
             torch.cuda.synchronize()
             reset_context()
         self.graph_pool = pool

@@ -78,3 +78,25 @@ def test_silu_and_mul(dev, rows, inter):
     x = (torch.randn(rows, 2 * inter, generator=g) * 2).to(torch.bfloat16)
     out = layers.silu_and_mul(x.to(dev))
     assert_bf16_close(out, glue.silu_and_mul(x), "silu_and_mul", max_frac=0.01)
+
+
+def test_qk_norm_rope_fused_scatter_matches_store_kvcache(dev):
+    """The fused kernel writes to the cache exactly what store_kvcache writes from its outputs."""
+    import nanovllm_amd as nva
+    g = torch.Generator().manual_seed(21)
+    n, hq, hkv, d = 300, 16, 8, 128
+    qkv = torch.randn(n, (hq + 2 * hkv) * d, generator=g).to(torch.bfloat16).to(dev)
+    w = (1 + 0.2 * torch.randn(d, generator=g)).to(torch.bfloat16).to(dev)
+    pos = torch.randint(0, 4096, (n,), generator=g).to(dev)
+    cache = layers.build_rope_cache(d, 4096, 1e6, dev)
+    slots = torch.randperm(4 * 256, generator=g)[:n].to(torch.int32)
+    slots[::7] = -1
+    slots = slots.to(dev)
+    kc1, vc1 = (torch.zeros(4, 256, hkv, d, dtype=torch.bfloat16, device=dev) for _ in range(2))
+    kc2, vc2 = torch.zeros_like(kc1), torch.zeros_like(vc1)
+    q1, k1, v1 = layers.qk_norm_rope(qkv, pos, w, w, cache, hq, hkv, d, 1e-6, kv_store=(kc1, vc1, slots))
+    q2, k2, v2 = layers.qk_norm_rope(qkv, pos, w, w, cache, hq, hkv, d, 1e-6)
+    nva.store_kvcache(k2, v2, kc2, vc2, slots)
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q2) and torch.equal(k1, k2)
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2) and bool(kc1.any()) and bool(vc1.any())
