@@ -10,6 +10,7 @@ already resident in HBM.  Workloads (shapes are the BASELINE.json configs):
     scatter   store_kvcache, 4096 tokens into 512 blocks x 256 slots              (config 1)
     prefill   causal varlen prefill, 16 sequences, half with cached prefix        (config 3)
     sampler   temperature sampling over 256 x 151,936 logits
+    decode-e2e-shape / copy   profiling helpers: the roofline leg of e2e alone; a plain copy of known size
 The line carries `roofline` (algorithmic bytes or flops of the dominant kernel per launch,
 divided by its average duration measured with HIP events on the launch stream) and
 `cpu_baseline` (the CPU oracle timed on this box's host cores on a bounded sample).
@@ -90,7 +91,7 @@ def bench_decode(args, dev):
                    "batch": 64, "kv_tokens_per_step": tokens},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "decode_split_kernel<2> + decode_merge_kernel",
+                     "kernel": "decode_stream_kernel<2> + decode_merge_kernel<2>",
                      "algorithmic_bytes_per_launch": int(mean_alg)},
     }
 
@@ -227,6 +228,75 @@ def e2e_workload(num_seqs=256, max_input_len=1024, max_output_len=1024, vocab=15
     return prompts, params
 
 
+# HBM bytes per launch of decode_stream_kernel<2> at the e2e decode shape, from two rocprofv3 --pmc
+# passes of `bench.py --workload decode-e2e-shape` (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each
+# scaled by what the same counter reads for the plain copy kernel of `--workload copy` (known size).
+MEASURED_TRAFFIC_E2E_SHAPE = 874_900_000      # stream kernel 869.9 MB + merge kernel 5.0 MB (algorithmic: 855.3 MB)
+
+
+def decode_e2e_shape_roofline(dev, caches, num_blocks):
+    """Paged decode attention at the e2e workload's own decode shape: the 256 requests of the bench
+    mix mid-flight (context = prompt + half of the output, mean 813 tokens), block tables drawn
+    without replacement from the pool, timed with HIP events while rotating through `caches`
+    (separate K/V pools, so neither L2 nor the 256 MB Infinity Cache can serve re-reads)."""
+    import torch
+    import nanovllm_amd as nva
+    from nanovllm_amd import synthetic
+    prompts, params = e2e_workload()
+    g = torch.Generator().manual_seed(1)
+    ctx = torch.tensor([len(p) + sp.max_tokens // 2 for p, sp in zip(prompts, params)], dtype=torch.int32)
+    tables = synthetic.decode_tables(ctx.tolist(), num_blocks, g, width=16).to(dev)
+    ctx_d = ctx.to(dev)
+    hq, hkv, dh = 16, caches[0][0].shape[2], caches[0][0].shape[3]
+    q = torch.randn(256, hq, dh, device=dev).to(torch.bfloat16)
+    out = torch.empty(256, 1, hq, dh, dtype=torch.bfloat16, device=dev)
+    scale = dh ** -0.5
+    fns = [lambda kc=kc, vc=vc: nva.paged_decode_attention(q, kc, vc, ctx_d, tables, scale, out=out)
+           for kc, vc in caches]
+    reps = max(5 * len(fns), 60)
+    ms = _event_time_ms(fns, reps, len(fns)) / reps
+    alg = int(ctx.sum()) * hkv * dh * 2 * 2 + 2 * q.numel() * 2
+    gbps = alg / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_E2E_SHAPE,
+            "kernel": "decode_stream_kernel<2> (+ decode_merge_kernel<2>): paged decode attention, batch 256, "
+                      "mean ctx %d" % int(ctx.float().mean()),
+            "algorithmic_bytes_per_launch": alg, "us_per_launch": round(ms * 1e3, 2)}
+
+
+def bench_decode_e2e_shape(args, dev):
+    """Only the roofline leg of the e2e workload (for profiling runs): 4 private 4096-block pools."""
+    import torch
+    caches = []
+    for p in range(4):
+        g = torch.Generator(device=dev).manual_seed(200 + p)
+        caches.append(tuple(torch.randn((4096, 256, 8, 128), generator=g, device=dev, dtype=torch.float32)
+                            .to(torch.bfloat16) for _ in range(2)))
+    roof = decode_e2e_shape_roofline(dev, caches, 4096)
+    result = {"metric": "paged decode attention at the e2e decode shape, achieved HBM GB/s", "value": roof["achieved"],
+              "unit": "GB/s", "ms_per_step": round(roof["us_per_launch"] / 1e3, 5),
+              "config": {"workload": "paged_decode_attn, batch 256, contexts of the e2e bench mix mid-flight, "
+                                     "4 rotating 4 GiB KV pools"}, "roofline": roof}
+    return result, (lambda: None)
+
+
+def bench_copy(args, dev):
+    """A plain device-to-device copy of known size: the calibration kernel for FETCH_SIZE / WRITE_SIZE."""
+    import torch
+    n = 256 << 20
+    src = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 255)
+    dsts = [torch.empty_like(src) for _ in range(3)]
+    ms = _event_time_ms([lambda d=d: d.copy_(src) for d in dsts], args.steps, args.warmup) / args.steps
+    gbps = 2 * n / (ms * 1e-3) / 1e9
+    result = {"metric": "plain copy kernel, read + write GB/s", "value": round(gbps, 1), "unit": "GB/s",
+              "ms_per_step": round(ms, 5),
+              "config": {"workload": "torch copy_ of 268,435,456 bytes (reads 256 MiB, writes 256 MiB)"},
+              "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": 2 * n, "kernel": "copy",
+                           "algorithmic_bytes_per_launch": 2 * n}}
+    return result, (lambda: None)
+
+
 def bench_e2e(args, dev):
     """Qwen3-0.6B architecture, random weights, 256 requests, hipGraph decode: output tok/s."""
     import torch
@@ -251,24 +321,8 @@ def bench_e2e(args, dev):
     assert all(len(o["token_ids"]) == p.max_tokens for o, p in zip(outs, params))
     tok_s = total_out * args.steps / dt
 
-    # roofline of the dominant kernel (paged decode attention) at this workload's own decode
-    # shape: 256 running sequences whose context lengths are prompt + half of the output, read
-    # through each of the 28 layers' caches in turn (7.5 GB apart, so nothing is cache-resident)
-    from nanovllm_amd import synthetic
-    g = torch.Generator().manual_seed(1)
-    full_prompts, full_params = e2e_workload()
-    ctx = torch.tensor([len(p) + sp.max_tokens // 2 for p, sp in zip(full_prompts, full_params)], dtype=torch.int32)
-    tables = synthetic.decode_tables(ctx.tolist(), llm.config.num_kvcache_blocks, g, width=16).to(dev)
-    ctx_d = ctx.to(dev)
-    q = torch.randn(256, model.num_attention_heads, model.head_dim, device=dev).to(torch.bfloat16)
-    out = torch.empty(256, 1, model.num_attention_heads, model.head_dim, dtype=torch.bfloat16, device=dev)
     layers = [m for m in llm.model_runner.model.modules() if isinstance(m, nva.Attention)]
-    fns = [lambda a=a: nva.paged_decode_attention(q, a.k_cache, a.v_cache, ctx_d, tables, a.scale, out=out)
-           for a in layers]
-    reps = 5 * len(fns)
-    ms = _event_time_ms(fns, reps, len(fns)) / reps
-    alg = int(ctx.sum()) * model.num_key_value_heads * model.head_dim * 2 * 2 + 2 * q.numel() * 2
-    gbps = alg / (ms * 1e-3) / 1e9
+    roof = decode_e2e_shape_roofline(dev, [(a.k_cache, a.v_cache) for a in layers], llm.config.num_kvcache_blocks)
     st = llm.stats
     result = {
         "metric": "output tok/s, Qwen3-0.6B bench shape; decode-attn HBM GB/s vs ~8 TB/s",
@@ -278,11 +332,7 @@ def bench_e2e(args, dev):
                                "U[100,1024], temperature 0.6, ignore_eos, " + ("eager" if args.eager else "hipGraph decode"),
                    "requests": 256, "output_tokens": total_out, "engine_steps_per_pass": (st["prefill_steps"] + st["decode_steps"]) // args.steps,
                    "prefill_s_per_pass": round(st["prefill_s"] / args.steps, 3), "decode_s_per_pass": round(st["decode_s"] / args.steps, 3)},
-        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "decode_stream_kernel<2> + decode_merge_kernel<2> (paged decode attention, batch 256, "
-                               "mean ctx %d)" % int(ctx.float().mean()),
-                     "algorithmic_bytes_per_launch": alg, "us_per_launch": round(ms * 1e3, 2)},
+        "roofline": roof,
     }
 
     def cpu():
@@ -291,8 +341,8 @@ def bench_e2e(args, dev):
     return result, cpu
 
 
-WORKLOADS = {"e2e": bench_e2e, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
-DEFAULT_STEPS = {"e2e": 1, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
+WORKLOADS = {"e2e": bench_e2e, "decode-e2e-shape": bench_decode_e2e_shape, "copy": bench_copy, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
+DEFAULT_STEPS = {"e2e": 1, "decode-e2e-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
 
 
 def main():
@@ -331,7 +381,9 @@ def main():
         "data": "synthetic", "config": result["config"], "roofline": result["roofline"],
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_fn()
+        base = cpu_fn()
+        if base is not None:
+            line["cpu_baseline"] = base
     print(json.dumps(line), flush=True)
 
 
