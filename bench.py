@@ -6,6 +6,7 @@
 A "step" is one pass of the selected workload over one batch of synthetic input that is
 already resident in HBM.  Workloads (shapes are the BASELINE.json configs):
     e2e       (default) generate() over 256 requests on a Qwen3-0.6B-architecture model (config 4)
+    longctx   Qwen3-8B-architecture long-context decode stress, batch 128, ctx U[4096,16384]  (config 5)
     decode    paged decode attention, batch 64, 16/8 heads, ctx U[100,2048]       (config 2)
     scatter   store_kvcache, 4096 tokens into 512 blocks x 256 slots              (config 1)
     prefill   causal varlen prefill, 16 sequences, half with cached prefix        (config 3)
@@ -341,8 +342,89 @@ def bench_e2e(args, dev):
     return result, cpu
 
 
-WORKLOADS = {"e2e": bench_e2e, "decode-e2e-shape": bench_decode_e2e_shape, "copy": bench_copy, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
-DEFAULT_STEPS = {"e2e": 1, "decode-e2e-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
+def bench_longctx(args, dev):
+    """Long-context decode stress (config 5): Qwen3-8B architecture, batch 128, contexts U[4096,16384],
+    256-token KV blocks scattered randomly over a cache sized to the drawn contexts, 128 decode steps,
+    even requests greedy and odd requests at temperature 1.0.  The prompts' KV is synthetic (the
+    cache is filled with N(0,1) noise and the sequences are placed directly), so only the decode
+    phase is run and timed; a step = one pass of 128 engine decode steps."""
+    import random
+    import torch
+    from nanovllm_amd.engine import SamplingParams, Sequence, SequenceStatus, qwen3_8b
+    from nanovllm_amd.engine.llm import LLM
+    model = qwen3_8b()
+    rng = random.Random(0)
+    n_req, n_steps = args.requests if args.requests != 256 else 128, 128
+    ctx = [rng.randint(4096, 16384) for _ in range(n_req)]
+    need = sum(-(-(c + n_steps) // 256) for c in ctx)
+    llm = LLM(model, enforce_eager=args.eager, max_model_len=16384 + 256, max_num_batched_tokens=32768,
+              max_num_seqs=n_req, num_kvcache_blocks=need + 8)
+    mr, sch = llm.model_runner, llm.scheduler
+    with torch.inference_mode():
+        for l in range(model.num_hidden_layers):                 # synthetic KV content
+            mr.kv_cache[0, l].normal_()
+            mr.kv_cache[1, l].normal_()
+    torch.cuda.synchronize()
+
+    def place():
+        free = list(range(llm.config.num_kvcache_blocks))
+        rng.shuffle(free)                                        # blocks scattered randomly over the cache
+        bm = sch.block_manager
+        seqs = []
+        for i, c in enumerate(ctx):
+            s = Sequence([rng.randint(0, model.vocab_size - 1) for _ in range(c)],
+                         SamplingParams(temperature=0.0 if i % 2 == 0 else 1.0, max_tokens=n_steps, ignore_eos=True))
+            # the state a real prefill leaves behind: blocks for the first c-1 tokens (the scheduler adds the
+            # block of the token being decoded), full blocks sealed with their chained hash
+            for _ in range(-(-(c - 1) // 256)):
+                blk = bm._take(free.pop())
+                s.block_table.append(blk.block_id)
+            for j in range((c - 1) // 256):
+                blk = bm.blocks[s.block_table[j]]
+                blk.hash = bm.compute_hash(s.block(j), bm.blocks[s.block_table[j - 1]].hash if j else -1)
+                blk.token_ids = s.block(j)
+            s.num_prompt_tokens = len(s)
+            s.status = SequenceStatus.RUNNING
+            sch.running.append(s)
+            seqs.append(s)
+        return seqs
+
+    def one_pass():
+        seqs = place()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        steps = 0
+        while not llm.is_finished():
+            llm.step()
+            steps += 1
+        torch.cuda.synchronize()
+        assert steps == n_steps and all(s.num_completion_tokens == n_steps for s in seqs)
+        return time.perf_counter() - t0
+
+    for _ in range(args.warmup):
+        one_pass()
+    dt = sum(one_pass() for _ in range(args.steps)) / args.steps
+    tok_s = n_req * n_steps / dt
+    kv_bytes_per_step = sum(c + n_steps // 2 for c in ctx) * model.num_hidden_layers * model.num_key_value_heads * model.head_dim * 2 * 2
+    result = {
+        "metric": "output tok/s, Qwen3-8B long-context decode (config 5)", "value": round(tok_s, 1), "unit": "tok/s",
+        "ms_per_step": round(dt * 1e3, 2),
+        "config": {"workload": "long-context decode: Qwen3-8B architecture (36 layers, hidden 4096, 32q/8kv heads x 128, "
+                               "MLP 12288, random bf16 weights), batch %d, contexts U[4096,16384] (mean %d), synthetic KV in "
+                               "%d randomly scattered 256-token blocks (%.1f GB cache), 128 decode steps, greedy + T=1.0, %s"
+                               % (n_req, sum(ctx) // n_req, need, (need + 8) * 37.75e6 / 1e9,
+                                  "eager" if args.eager else "hipGraph decode"),
+                   "ms_per_decode_step": round(dt / n_steps * 1e3, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(kv_bytes_per_step / (dt / n_steps) / 1e9, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(kv_bytes_per_step / (dt / n_steps) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "whole decode step (36 x decode_stream_kernel<4> dominate): KV bytes of one step / step time",
+                     "algorithmic_bytes_per_launch": kv_bytes_per_step},
+    }
+    return result, (lambda: None)
+
+
+WORKLOADS = {"e2e": bench_e2e, "longctx": bench_longctx, "decode-e2e-shape": bench_decode_e2e_shape, "copy": bench_copy, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
+DEFAULT_STEPS = {"e2e": 1, "longctx": 1, "decode-e2e-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
 
 
 def main():
@@ -362,7 +444,7 @@ def main():
     if args.steps is None:
         args.steps = DEFAULT_STEPS[args.workload]
     if args.warmup is None:
-        args.warmup = 1 if args.workload == "e2e" else max(3, args.steps // 10)
+        args.warmup = 1 if args.workload in ("e2e", "longctx") else max(3, args.steps // 10)
 
     import torch
     if not torch.cuda.is_available():
