@@ -398,7 +398,7 @@ def bench_longctx(args, dev):
             llm.step()
             steps += 1
         torch.cuda.synchronize()
-        assert steps == n_steps and all(s.num_completion_tokens == n_steps for s in seqs)
+        assert steps in (n_steps, n_steps + 1) and all(s.num_completion_tokens == n_steps for s in seqs)   # +1: the last tokens are read back
         return time.perf_counter() - t0
 
     for _ in range(args.warmup):

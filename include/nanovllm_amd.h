@@ -194,6 +194,16 @@ int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const int64_t *pos
 int nva_silu_and_mul(const void *x, int64_t x_row_stride, void *out,
                      int32_t rows, int32_t inter, void *stream);
 
+/*
+ * Feeds the tokens sampled by one decode step to the next one without a trip through the host:
+ * input_ids[i] = prev_tokens[src_index[i]] where 0 <= src_index[i] < n_prev, else unchanged.
+ * It stands where the reference copies last_token of every sequence from the host
+ * (nanovllm/engine/model_runner.py:166,173); rows whose token the host already knows carry -1.
+ * input_ids: int64 [n], src_index: int32 [n], prev_tokens: int64 [n_prev] (the sampler's output).
+ */
+int nva_gather_tokens(int64_t *input_ids, const int32_t *src_index, const int64_t *prev_tokens,
+                      int32_t n, int32_t n_prev, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -149,6 +149,14 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const bf16_t *__restr
     *reinterpret_cast<uint4 *>(out + row * inter + e) = o;
 }
 
+// input_ids[i] = prev_tokens[src_index[i]] for rows that name a row of the previous step
+__global__ void gather_tokens_kernel(int64_t *ids, const int32_t *src, const int64_t *prev, int32_t n, int32_t n_prev) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int32_t j = src[i];
+    if (static_cast<uint32_t>(j) < static_cast<uint32_t>(n_prev)) ids[i] = prev[j];
+}
+
 }  // namespace nva
 
 extern "C" int nva_rms_norm(const void *x, int64_t x_row_stride, const void *residual, int64_t residual_row_stride,
@@ -216,5 +224,16 @@ extern "C" int nva_silu_and_mul(const void *x, int64_t x_row_stride, void *out, 
     hipLaunchKernelGGL(silu_and_mul_kernel, dim3(static_cast<uint32_t>((total + 255) / 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const bf16_t *>(x), x_row_stride,
                        static_cast<bf16_t *>(out), total, chunks_per_row, inter);
+    return launch_status();
+}
+
+extern "C" int nva_gather_tokens(int64_t *input_ids, const int32_t *src_index, const int64_t *prev_tokens, int32_t n,
+                                 int32_t n_prev, void *stream) {
+    using namespace nva;
+    if (n < 0 || n_prev < 0) return NVA_ERR_BAD_SHAPE;
+    if (n == 0 || n_prev == 0) return NVA_OK;
+    if (!input_ids || !src_index || !prev_tokens) return NVA_ERR_NULL_POINTER;
+    hipLaunchKernelGGL(gather_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       input_ids, src_index, prev_tokens, n, n_prev);
     return launch_status();
 }

@@ -10,12 +10,12 @@ block has not been handed out again.
 from __future__ import annotations
 
 from collections import deque
-from typing import Deque, Dict, List, Set
+from typing import Deque, Dict, List, Optional, Set
 
 import numpy as np
 import xxhash
 
-from .sequence import Sequence
+from .sequence import PENDING_TOKEN, Sequence
 
 NO_HASH = -1
 
@@ -116,11 +116,24 @@ class BlockManager:
             assert last.hash != NO_HASH
             table.append(self._take(self.free_block_ids[0]).block_id)
         elif fill == 0:                            # block completed by the last token: seal it
-            assert last.hash == NO_HASH
-            ids = seq.block(seq.num_blocks - 1)
-            prefix = self.blocks[table[-2]].hash if len(table) > 1 else NO_HASH
-            last.hash = self.compute_hash(ids, prefix)
-            last.token_ids = ids
-            self.hash_to_block_id[last.hash] = last.block_id
+            if seq.token_ids[-1] != PENDING_TOKEN:
+                self.seal(seq, seq.num_blocks - 1)
         else:
             assert last.hash == NO_HASH
+
+    def seal(self, seq: Sequence, index: int, table: Optional[List[int]] = None) -> None:
+        """Register the content hash of the full block ``index`` of ``seq`` (no-op when it is
+        sealed already).  ``may_append`` does this when the block fills up; when the step loop
+        runs ahead of the sampled tokens the block's last id is not known at that moment, and the
+        loop seals the block once the token has been read back (``table``: the block table the
+        sequence had, if it has been deallocated since)."""
+        table = seq.block_table if table is None else table
+        blk = self.blocks[table[index]]
+        if blk.hash != NO_HASH:
+            return
+        ids = seq.block(index)
+        assert len(ids) == self.block_size and PENDING_TOKEN not in ids[-2:]
+        prefix = self.blocks[table[index - 1]].hash if index > 0 else NO_HASH
+        blk.hash = self.compute_hash(ids, prefix)
+        blk.token_ids = ids
+        self.hash_to_block_id[blk.hash] = blk.block_id

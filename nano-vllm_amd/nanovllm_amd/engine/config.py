@@ -69,6 +69,7 @@ class EngineConfig:
     kvcache_block_size: int = 256
     num_kvcache_blocks: int = -1
     seed: int = 0
+    decode_lookahead: bool = True                        # launch decode steps one step ahead of their tokens
 
     def __post_init__(self):
         if isinstance(self.model, ModelConfig):

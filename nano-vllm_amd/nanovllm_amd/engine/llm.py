@@ -28,6 +28,10 @@ class LLMEngine:
             config.eos = tokenizer.eos_token_id
         self.model_runner = ModelRunner(config)
         self.scheduler = Scheduler(config)
+        # Decode steps are launched one step ahead of their tokens: while the GPU runs step t the
+        # host reads the tokens of step t-1, retires finished sequences and prepares step t+1.
+        self.lookahead = config.decode_lookahead and not config.enforce_eager
+        self._inflight = None                       # (DecodeHandle, token positions) not yet committed
         self.stats = {"prefill_steps": 0, "decode_steps": 0, "prefill_tokens": 0, "decode_tokens": 0,
                       "prefill_s": 0.0, "decode_s": 0.0}
 
@@ -39,20 +43,49 @@ class LLMEngine:
         self.scheduler.add(Sequence(prompt, sampling_params))
 
     def step(self):
+        """One scheduling iteration.  Returns ``([(seq_id, completion ids) of finished requests],
+        tokens processed: positive for prefill, negative for decode)`` like the reference's
+        ``LLMEngine.step`` (llm_engine.py:48-54); with lookahead a request is reported when its
+        last token has been read back, one iteration after the step that sampled it."""
         t0 = perf_counter()
-        seqs, is_prefill = self.scheduler.schedule()
-        token_ids = self.model_runner.run(seqs, is_prefill)
-        self.scheduler.postprocess(seqs, token_ids)
-        outputs = [(s.seq_id, s.completion_token_ids) for s in seqs if s.is_finished]
+        sch, runner = self.scheduler, self.model_runner
+        finished = []
+        # admission (prefix hashes, recompute of preempted sequences) needs every token in place
+        if self._inflight is not None and (sch.waiting or not sch.running):
+            finished += self._commit_inflight()
+        if sch.is_finished():
+            return self._report(finished), 0
+        seqs, is_prefill = sch.schedule()
+        if not is_prefill and self.lookahead and runner.can_launch_ahead(len(seqs)):
+            handle = runner.launch_decode(seqs, self._inflight[0] if self._inflight else None)
+            where = sch.advance(seqs)
+            if self._inflight is not None:
+                finished += self._commit_inflight()
+            self._inflight = (handle, where)
+        else:
+            if self._inflight is not None:          # a decode batch beyond the captured sizes
+                finished += self._commit_inflight()
+            token_ids = runner.run(seqs, is_prefill)
+            sch.postprocess(seqs, token_ids)
+            finished += [s for s in seqs if s.is_finished]
         num_tokens = sum(len(s) for s in seqs) if is_prefill else -len(seqs)
         kind = "prefill" if is_prefill else "decode"
         self.stats[kind + "_steps"] += 1
         self.stats[kind + "_tokens"] += abs(num_tokens)
         self.stats[kind + "_s"] += perf_counter() - t0
-        return outputs, num_tokens
+        return self._report(finished), num_tokens
+
+    def _commit_inflight(self):
+        handle, where = self._inflight
+        self._inflight = None
+        return self.scheduler.commit(handle.seqs, where, handle.tokens())
+
+    @staticmethod
+    def _report(seqs):
+        return [(s.seq_id, s.completion_token_ids) for s in seqs]
 
     def is_finished(self) -> bool:
-        return self.scheduler.is_finished()
+        return self.scheduler.is_finished() and self._inflight is None
 
     def generate(self, prompts, sampling_params, use_tqdm: bool = False):
         if not isinstance(sampling_params, list):

@@ -8,16 +8,32 @@ with numpy into pinned staging buffers instead of Python lists.
 """
 from __future__ import annotations
 
-from typing import List, Optional
+from dataclasses import dataclass
+from typing import Dict, List, Optional
 
 import numpy as np
 import torch
 
+from .. import _lib
 from ..context import reset_context, set_context
 from ..sampler import Sampler
 from .config import EngineConfig
 from .model import Qwen3ForCausalLM
-from .sequence import Sequence
+from .sequence import PENDING_TOKEN, Sequence
+
+
+@dataclass
+class DecodeHandle:
+    """A decode step that has been enqueued but whose tokens have not been read back."""
+    seqs: List[Sequence]
+    row_of: Dict[int, int]                # seq_id -> row of the step's batch
+    tokens_dev: torch.Tensor              # int64 [len(seqs)], the sampler's output
+    tokens_host: torch.Tensor             # pinned copy, valid once ``ready`` has completed
+    ready: torch.cuda.Event
+
+    def tokens(self) -> List[int]:
+        self.ready.synchronize()
+        return self.tokens_host[: len(self.seqs)].tolist()
 
 
 def build_block_tables(seqs: List[Sequence]) -> np.ndarray:
@@ -162,34 +178,48 @@ class ModelRunner:
 
     # ---- execution -----------------------------------------------------------------------------
     def _init_decode_staging(self, max_bs: int) -> None:
-        """One pinned host buffer and one device buffer holding every per-step decode input; the
+        """Pinned host buffers and one device buffer holding every per-step decode input; the
         graph's static tensors are typed views into the device buffer, so a decode step needs a
         single host-to-device copy (the reference issues one copy per tensor plus one device copy
-        per graph variable, nanovllm/engine/model_runner.py:162-179,197-203)."""
+        per graph variable, nanovllm/engine/model_runner.py:162-179,197-203).  There are two host
+        buffers, used in turn: with steps launched ahead of the previous step's tokens the copy
+        of one step may still be queued while the host fills in the next."""
         fields = [("input_ids", np.int64, (max_bs,)), ("positions", np.int64, (max_bs,)),
                   ("slot_mapping", np.int32, (max_bs,)), ("context_lens", np.int32, (max_bs,)),
-                  ("temperatures", np.float32, (max_bs,)), ("block_tables", np.int32, (max_bs, self.max_table_width))]
+                  ("temperatures", np.float32, (max_bs,)), ("token_src", np.int32, (max_bs,)),
+                  ("block_tables", np.int32, (max_bs, self.max_table_width))]
         offsets, total = {}, 0
         for name, dt, shape in fields:
             nbytes = int(np.prod(shape)) * np.dtype(dt).itemsize
             offsets[name] = (total, nbytes, dt, shape)
             total += (nbytes + 255) // 256 * 256
         # zero-filled: rows past the batch are replayed too (bucket padding) and must hold valid ids / positions
-        self._stage_host = torch.zeros(total, dtype=torch.uint8).pin_memory()
+        self._stage_host = [torch.zeros(total, dtype=torch.uint8).pin_memory() for _ in range(2)]
         self._stage_dev = torch.zeros(total, dtype=torch.uint8, device=self.device)
-        host_np = self._stage_host.numpy()
+        self._tokens_host = [torch.zeros(max_bs, dtype=torch.int64).pin_memory() for _ in range(2)]
+        self._stage_turn = 0
         tdt = {np.int64: torch.int64, np.int32: torch.int32, np.float32: torch.float32}
-        self._stage_np, self.graph_vars = {}, {}
+        self._stage_np, self.graph_vars = [{}, {}], {}
         for name, (off, nbytes, dt, shape) in offsets.items():
-            self._stage_np[name] = host_np[off: off + nbytes].view(dt).reshape(shape)
+            for k in range(2):
+                self._stage_np[k][name] = self._stage_host[k].numpy()[off: off + nbytes].view(dt).reshape(shape)
             self.graph_vars[name] = self._stage_dev[off: off + nbytes].view(tdt[dt]).view(shape)
 
-    def _run_decode_graph(self, seqs: List[Sequence]) -> torch.Tensor:
-        """Fill the staging buffer, copy it once, replay the bucket's graph; returns logits."""
+    def _run_decode_graph(self, seqs: List[Sequence], prev: Optional[DecodeHandle] = None) -> torch.Tensor:
+        """Fill a staging buffer, copy it once, replay the bucket's graph; returns logits.  Rows
+        whose last token is still pending take it on the device from ``prev``'s sampler output."""
         bs = len(seqs)
         bucket = next(x for x in self.graph_bs if x >= bs)
         h = build_decode_inputs(seqs, self.block_size)
-        st = self._stage_np
+        self._stage_turn ^= 1
+        st = self._stage_np[self._stage_turn]
+        pending = h["input_ids"] == PENDING_TOKEN
+        n_pending = int(pending.sum())
+        if n_pending:
+            assert prev is not None, "a pending token needs the step that samples it"
+            st["token_src"][:bs] = np.fromiter((prev.row_of[s.seq_id] if p else -1 for s, p in zip(seqs, pending)),
+                                               dtype=np.int32, count=bs)
+            h["input_ids"][pending] = 0
         st["input_ids"][:bs] = h["input_ids"]
         st["positions"][:bs] = h["positions"]
         st["slot_mapping"][:bs] = h["slot_mapping"]
@@ -198,10 +228,33 @@ class ModelRunner:
         st["context_lens"][bs:bucket] = 0                         # ... and attend over nothing
         st["temperatures"][:bs] = np.fromiter((s.temperature for s in seqs), dtype=np.float32, count=bs)
         st["block_tables"][:bs, : h["block_tables"].shape[1]] = h["block_tables"]   # stale columns stay: never read
-        self._stage_dev.copy_(self._stage_host, non_blocking=True)
+        self._stage_dev.copy_(self._stage_host[self._stage_turn], non_blocking=True)
+        if n_pending:
+            gv = self.graph_vars
+            rc = _lib.load().nva_gather_tokens(gv["input_ids"].data_ptr(), gv["token_src"].data_ptr(),
+                                               prev.tokens_dev.data_ptr(), bs, prev.tokens_dev.numel(),
+                                               torch.cuda.current_stream().cuda_stream)
+            _lib.check(rc, "nva_gather_tokens")
         for graph in self.graphs[bucket]:                         # later segments are enqueued while the first runs
             graph.replay()
         return self.model.compute_logits(self.graph_vars["outputs"][:bs])
+
+    def can_launch_ahead(self, num_seqs: int) -> bool:
+        """Whether a decode batch of this size can be launched without waiting for its tokens."""
+        return bool(self.graph_bs) and num_seqs <= self.graph_bs[-1]
+
+    def launch_decode(self, seqs: List[Sequence], prev: Optional[DecodeHandle] = None) -> DecodeHandle:
+        """Enqueue one decode step and its sampling; nothing is read back.  ``prev`` is the step
+        launched before, if its tokens have not been committed to the sequences yet."""
+        with torch.inference_mode():
+            logits = self._run_decode_graph(seqs, prev)
+            tokens_dev = self.sampler(logits, self.graph_vars["temperatures"][: len(seqs)])
+            tokens_host = self._tokens_host[self._stage_turn]
+            tokens_host[: len(seqs)].copy_(tokens_dev, non_blocking=True)
+            ready = torch.cuda.Event()
+            ready.record()
+        reset_context()
+        return DecodeHandle(seqs, {s.seq_id: i for i, s in enumerate(seqs)}, tokens_dev, tokens_host, ready)
 
     @torch.inference_mode()
     def run_model(self, input_ids: torch.Tensor, positions: torch.Tensor, is_prefill: bool) -> torch.Tensor:

@@ -12,7 +12,7 @@ from typing import Deque, List, Tuple
 
 from .block_manager import BlockManager
 from .config import EngineConfig
-from .sequence import Sequence, SequenceStatus
+from .sequence import PENDING_TOKEN, Sequence, SequenceStatus
 
 
 class Scheduler:
@@ -77,3 +77,56 @@ class Scheduler:
                 seq.status = SequenceStatus.FINISHED
                 self.block_manager.deallocate(seq)
                 self.running.remove(seq)
+
+    # ---- running one step ahead of the sampled tokens ---------------------------------------------
+    # ``postprocess`` needs the tokens of a step before the next one can be scheduled, which leaves
+    # the GPU idle while the host reads them back and prepares the next batch.  ``advance`` +
+    # ``commit`` split it in two: ``advance`` does everything that depends on lengths only (it
+    # appends a PENDING_TOKEN and retires sequences that reach max_tokens), so that the next
+    # decode step can be scheduled and launched at once; ``commit`` fills in the tokens when they
+    # arrive, ends sequences that sampled eos (their one speculative step is dropped) and seals
+    # the blocks those tokens completed.  With every step committed, the state equals what
+    # ``postprocess`` leaves, except that blocks freed by an eos come back one step later.
+    def advance(self, seqs: List[Sequence]) -> List[int]:
+        """Returns the index in ``token_ids`` that the step's token of every sequence will take."""
+        where = []
+        for seq in seqs:
+            where.append(len(seq))
+            seq.append_token(PENDING_TOKEN)
+            if seq.num_completion_tokens == seq.max_tokens:
+                bs = self.block_manager.block_size
+                if len(seq) >= 2 and seq.token_ids[-2] == PENDING_TOKEN and (len(seq) - 1) % bs == 0:
+                    # the previous, uncommitted token completed a block: commit seals it from this copy
+                    seq.late_seal = (len(seq) - 2, list(seq.block_table))
+                seq.status = SequenceStatus.FINISHED
+                self.block_manager.deallocate(seq)
+                self.running.remove(seq)
+        return where
+
+    def commit(self, seqs: List[Sequence], where: List[int], token_ids: List[int]) -> List[Sequence]:
+        """Returns the sequences whose last token this was."""
+        done = []
+        for seq, at, tok in zip(seqs, where, token_ids):
+            if at >= len(seq):                     # dropped: the sequence ended on an earlier eos
+                continue
+            assert seq.token_ids[at] == PENDING_TOKEN
+            seq.token_ids[at] = int(tok)
+            hit_eos = (not seq.ignore_eos) and tok == self.eos
+            late_seal = seq.__dict__.pop("late_seal", None) if seq.is_finished else None
+            if late_seal is not None and late_seal[0] == at and not hit_eos:
+                self.block_manager.seal(seq, at // self.block_manager.block_size, late_seal[1])
+            if hit_eos and at + 1 < len(seq):
+                del seq.token_ids[at + 1:]         # drop the step that ran past the eos
+            if hit_eos and not seq.is_finished:
+                if seq.status is SequenceStatus.RUNNING:
+                    self.block_manager.deallocate(seq)
+                    self.running.remove(seq)
+                else:                              # preempted in the meantime: holds no blocks
+                    self.waiting.remove(seq)
+                seq.status = SequenceStatus.FINISHED
+            if seq.is_finished:
+                if at == len(seq) - 1:
+                    done.append(seq)
+            elif (at + 1) % self.block_manager.block_size == 0 and seq.block_table:
+                self.block_manager.seal(seq, at // self.block_manager.block_size)
+        return done

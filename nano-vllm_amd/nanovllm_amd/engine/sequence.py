@@ -13,6 +13,9 @@ from typing import List
 from .sampling_params import SamplingParams
 
 
+PENDING_TOKEN = -1          # stands in token_ids for a token that is sampled but not yet read back
+
+
 class SequenceStatus(enum.Enum):
     WAITING = enum.auto()
     RUNNING = enum.auto()

@@ -179,3 +179,107 @@ def test_engine_config_checks():
         SamplingParams(temperature=1e-12)
     assert SamplingParams(temperature=0).temperature == 0
     assert _config(max_model_len=10 ** 6, max_num_batched_tokens=65536).max_model_len == 40960
+
+
+# ---- decode steps launched one step ahead of their tokens --------------------------------------
+class _FakeHandle:
+    def __init__(self, seqs, toks):
+        self.seqs, self._toks = seqs, toks
+        self.row_of = {s.seq_id: i for i, s in enumerate(seqs)}
+
+    def tokens(self):
+        return self._toks
+
+
+class _FakeRunner:
+    """Stands in for the GPU: the token after a sequence of length n whose last token is t is a
+    fixed function of (first prompt token, n, t), so that any mix-up of rows, positions or
+    pending tokens changes the completions."""
+    vocab = 50
+
+    def __init__(self):
+        self.launched_ahead = 0
+
+    def _next(self, seq, last):
+        return (seq.token_ids[0] * 31 + len(seq) * 7 + last * 13) % self.vocab
+
+    def run(self, seqs, is_prefill):
+        from nanovllm_amd.engine.sequence import PENDING_TOKEN
+        assert all(PENDING_TOKEN not in s.token_ids for s in seqs)
+        return [self._next(s, s.token_ids[-1]) for s in seqs]
+
+    def can_launch_ahead(self, n):
+        return True
+
+    def launch_decode(self, seqs, prev=None):
+        from nanovllm_amd.engine.sequence import PENDING_TOKEN
+        toks = []
+        for s in seqs:
+            last = s.token_ids[-1]
+            if last == PENDING_TOKEN:
+                last = prev.tokens()[prev.row_of[s.seq_id]]
+                self.launched_ahead += 1
+            assert PENDING_TOKEN not in s.token_ids[:-1]
+            toks.append(self._next(s, last))
+        return _FakeHandle(list(seqs), toks)
+
+
+def _fake_engine(lookahead, **kw):
+    from nanovllm_amd.engine.llm import LLMEngine
+    eng = LLMEngine.__new__(LLMEngine)
+    eng.config = _config(**kw)
+    eng.tokenizer = None
+    eng.model_runner = _FakeRunner()
+    eng.scheduler = Scheduler(eng.config)
+    eng.lookahead = lookahead
+    eng._inflight = None
+    eng.stats = {k: 0 for k in ("prefill_steps", "decode_steps", "prefill_tokens", "decode_tokens", "prefill_s", "decode_s")}
+    return eng
+
+
+@pytest.mark.parametrize("eos,blocks", [(-1, 64), (7, 64), (-1, 9), (7, 9)])
+def test_lookahead_loop_matches_the_synchronous_loop(eos, blocks):
+    """Same completions with and without lookahead: plain, with sequences ending on eos (their
+    speculative step is dropped), with a cache so small that sequences are preempted and
+    recomputed, and both.  Lengths cross several block boundaries (sealing, new blocks)."""
+    rng = np.random.default_rng(3)
+    prompts = [[int(100 + i)] + rng.integers(0, 50, size=int(n)).tolist()
+               for i, n in enumerate(rng.integers(200, 700, size=12))]
+    params = [SamplingParams(max_tokens=int(m), ignore_eos=(eos < 0)) for m in rng.integers(1, 400, size=12)]
+    results, engines = [], []
+    for lookahead in (False, True):
+        eng = _fake_engine(lookahead, num_kvcache_blocks=blocks, eos=eos, max_num_batched_tokens=4096, max_model_len=4096)
+        results.append(eng.generate(prompts, params))
+        engines.append(eng)
+        bm = eng.scheduler.block_manager
+        assert len(bm.free_block_ids) == blocks and not bm.used_block_ids and eng._inflight is None
+    assert [r["token_ids"] for r in results[0]] == [r["token_ids"] for r in results[1]]
+    assert engines[1].model_runner.launched_ahead > 0 and engines[0].model_runner.launched_ahead == 0
+    for r, p in zip(results[1], params):
+        ids = r["token_ids"]
+        assert 1 <= len(ids) <= p.max_tokens and (len(ids) == p.max_tokens or ids[-1] == eos)
+        assert eos < 0 or eos not in ids[:-1]
+    if eos < 0 and blocks == 64:                                # no preemption, no eos: identical prefix-cache state
+        a, b = (e.scheduler.block_manager for e in engines)
+        assert a.hash_to_block_id == b.hash_to_block_id
+        assert [blk.hash for blk in a.blocks] == [blk.hash for blk in b.blocks]
+
+
+def test_commit_drops_the_step_that_ran_past_an_eos():
+    sch = Scheduler(_config(num_kvcache_blocks=4, eos=42))
+    a, b = _seq(10, max_tokens=8), _seq(10, 100, max_tokens=8)
+    sch.add(a)
+    sch.add(b)
+    batch, _ = sch.schedule()
+    sch.postprocess(batch, [1, 2])
+    batch, _ = sch.schedule()
+    w1 = sch.advance(batch)                                     # step t launched
+    batch2, _ = sch.schedule()
+    assert batch2 == [a, b]
+    w2 = sch.advance(batch2)                                    # step t+1 launched before t's tokens are known
+    assert len(a) == 13 and w1 == [11, 11] and w2 == [12, 12]
+    done = sch.commit(batch, w1, [42, 5])                       # a sampled eos at step t
+    assert done == [a] and a.completion_token_ids == [1, 42] and a.is_finished and not a.block_table
+    assert list(sch.running) == [b]
+    done = sch.commit(batch2, w2, [9, 6])                       # a's token of step t+1 is dropped
+    assert done == [] and a.completion_token_ids == [1, 42] and b.completion_token_ids == [2, 5, 6]

@@ -153,3 +153,36 @@ def test_preemption_by_recompute_still_finishes(dev):
     outs = llm.generate(prompts, params)                                     # 4 x 2 blocks needed, 6 exist
     assert [len(o["token_ids"]) for o in outs] == [p.max_tokens for p in params]
     assert llm.stats["prefill_steps"] > 1
+
+
+def test_lookahead_decode_produces_the_same_tokens(dev):
+    """Greedy requests with staggered output lengths (the batch shrinks, rows move) and lengths
+    that cross a block boundary: launching decode steps one step ahead of their tokens (ids
+    handed over on the device) gives exactly the tokens of the synchronous loop.  Then with an
+    eos token picked from that run, so that some requests end early and their speculative step is
+    dropped."""
+    prompts, params = _requests(12, seed=11, lo=200, hi=300, out_lo=3, out_hi=90, temperature=0.0)
+    runs = {}
+    for lookahead in (False, True):
+        llm = LLM(tiny_model(), max_model_len=2048, max_num_batched_tokens=4096, num_kvcache_blocks=40, max_num_seqs=16,
+                  decode_lookahead=lookahead)
+        assert llm.lookahead == lookahead
+        runs[lookahead] = [o["token_ids"] for o in llm.generate(prompts, params)]
+        assert len(llm.scheduler.block_manager.free_block_ids) == 40
+    assert runs[True] == runs[False]
+    eos = runs[False][0][len(runs[False][0]) // 2]              # a token the first request emits mid-way
+    for p in params:
+        p.ignore_eos = False
+    stopped = {}
+    for lookahead in (False, True):
+        llm = LLM(tiny_model(), max_model_len=2048, max_num_batched_tokens=4096, num_kvcache_blocks=40, max_num_seqs=16,
+                  decode_lookahead=lookahead, eos=eos)
+        stopped[lookahead] = [o["token_ids"] for o in llm.generate(prompts, params)]
+    # batches differ between the runs once sequences end early (other GEMM shapes, bf16 tie-breaks),
+    # so only the structure is compared: every request ends on its first eos or at max_tokens
+    for run in stopped.values():
+        for ids, p in zip(run, params):
+            assert 1 <= len(ids) <= p.max_tokens and eos not in ids[:-1]
+            assert ids[-1] == eos or len(ids) == p.max_tokens
+        assert any(ids[-1] == eos and len(ids) < p.max_tokens for ids, p in zip(run, params))
+    assert [r[:1] for r in stopped[True]] == [r[:1] for r in runs[True]]
