@@ -195,14 +195,20 @@ int nva_silu_and_mul(const void *x, int64_t x_row_stride, void *out,
                      int32_t rows, int32_t inter, void *stream);
 
 /*
- * Feeds the tokens sampled by one decode step to the next one without a trip through the host:
- * input_ids[i] = prev_tokens[src_index[i]] where 0 <= src_index[i] < n_prev, else unchanged.
- * It stands where the reference copies last_token of every sequence from the host
- * (nanovllm/engine/model_runner.py:166,173); rows whose token the host already knows carry -1.
- * input_ids: int64 [n], src_index: int32 [n], prev_tokens: int64 [n_prev] (the sampler's output).
+ * Brings the per-step decode inputs from a pinned host buffer into their device buffer with one
+ * kernel (the device reads host memory directly; no copy engine, no second launch), and feeds the
+ * tokens sampled by the previous step to this one without a trip through the host.  It stands
+ * where the reference copies input_ids, positions, slot_mapping, context_lens and block_tables
+ * from the host one by one (nanovllm/engine/model_runner.py:162-179,197-203).
+ *   dst[0 .. nbytes) = src_host[0 .. nbytes)                        (nbytes % 16 == 0, both 16-byte aligned)
+ *   then, with ids = (int64*)(dst + ids_offset) and idx = (int32*)(src_host + index_offset), for i < n:
+ *   ids[i] = prev_tokens[idx[i]] where 0 <= idx[i] < n_prev         (other rows keep the host's value)
+ * src_host must be device-accessible host memory (hipHostMalloc / a pinned torch tensor).
+ * prev_tokens: int64 [n_prev], the sampler's output of the previous step; NULL with n_prev == 0.
  */
-int nva_gather_tokens(int64_t *input_ids, const int32_t *src_index, const int64_t *prev_tokens,
-                      int32_t n, int32_t n_prev, void *stream);
+int nva_stage_decode_inputs(void *dst, const void *src_host, int64_t nbytes, int64_t ids_offset,
+                            int64_t index_offset, int32_t n, const int64_t *prev_tokens, int32_t n_prev,
+                            void *stream);
 
 #ifdef __cplusplus
 }

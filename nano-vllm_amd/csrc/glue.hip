@@ -149,12 +149,31 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const bf16_t *__restr
     *reinterpret_cast<uint4 *>(out + row * inter + e) = o;
 }
 
-// input_ids[i] = prev_tokens[src_index[i]] for rows that name a row of the previous step
-__global__ void gather_tokens_kernel(int64_t *ids, const int32_t *src, const int64_t *prev, int32_t n, int32_t n_prev) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const int32_t j = src[i];
-    if (static_cast<uint32_t>(j) < static_cast<uint32_t>(n_prev)) ids[i] = prev[j];
+// host staging buffer -> device buffer, 16 bytes per lane; the input ids that name a row of the
+// previous step's sampler output are taken from there instead
+__global__ void stage_decode_inputs_kernel(uint4 *dst, const uint4 *src, int64_t chunks, int64_t ids_chunk0,
+                                           const int32_t *index, int32_t n, const int64_t *prev, int32_t n_prev) {
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c >= chunks) return;
+    uint4 v = src[c];
+    const int64_t i0 = (c - ids_chunk0) * 2;                       // first of the two ids in this chunk
+    if (c >= ids_chunk0 && i0 < n) {
+        const int32_t j0 = index[i0];
+        if (static_cast<uint32_t>(j0) < static_cast<uint32_t>(n_prev)) {
+            const int64_t t = prev[j0];
+            v.x = static_cast<uint32_t>(t);
+            v.y = static_cast<uint32_t>(t >> 32);
+        }
+        if (i0 + 1 < n) {
+            const int32_t j1 = index[i0 + 1];
+            if (static_cast<uint32_t>(j1) < static_cast<uint32_t>(n_prev)) {
+                const int64_t t = prev[j1];
+                v.z = static_cast<uint32_t>(t);
+                v.w = static_cast<uint32_t>(t >> 32);
+            }
+        }
+    }
+    dst[c] = v;
 }
 
 }  // namespace nva
@@ -227,13 +246,23 @@ extern "C" int nva_silu_and_mul(const void *x, int64_t x_row_stride, void *out, 
     return launch_status();
 }
 
-extern "C" int nva_gather_tokens(int64_t *input_ids, const int32_t *src_index, const int64_t *prev_tokens, int32_t n,
-                                 int32_t n_prev, void *stream) {
+extern "C" int nva_stage_decode_inputs(void *dst, const void *src_host, int64_t nbytes, int64_t ids_offset,
+                                       int64_t index_offset, int32_t n, const int64_t *prev_tokens, int32_t n_prev,
+                                       void *stream) {
     using namespace nva;
-    if (n < 0 || n_prev < 0) return NVA_ERR_BAD_SHAPE;
-    if (n == 0 || n_prev == 0) return NVA_OK;
-    if (!input_ids || !src_index || !prev_tokens) return NVA_ERR_NULL_POINTER;
-    hipLaunchKernelGGL(gather_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       input_ids, src_index, prev_tokens, n, n_prev);
+    if (nbytes < 0 || n < 0 || n_prev < 0 || ids_offset < 0 || index_offset < 0) return NVA_ERR_BAD_SHAPE;
+    if (nbytes % 16 != 0 || ids_offset % 16 != 0 || index_offset % 4 != 0) return NVA_ERR_MISALIGNED;
+    if (ids_offset + static_cast<int64_t>(n) * 8 > nbytes || index_offset + static_cast<int64_t>(n) * 4 > nbytes)
+        return NVA_ERR_BAD_SHAPE;
+    if (nbytes == 0) return NVA_OK;
+    if (!dst || !src_host || (n_prev > 0 && !prev_tokens)) return NVA_ERR_NULL_POINTER;
+    if (!aligned16(dst) || !aligned16(src_host)) return NVA_ERR_MISALIGNED;
+    const int64_t chunks = nbytes / 16;
+    if ((chunks + 255) / 256 > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(stage_decode_inputs_kernel, dim3(static_cast<uint32_t>((chunks + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<uint4 *>(dst), static_cast<const uint4 *>(src_host),
+                       chunks, ids_offset / 16,
+                       reinterpret_cast<const int32_t *>(static_cast<const char *>(src_host) + index_offset), n,
+                       prev_tokens, n_prev);
     return launch_status();
 }

@@ -41,7 +41,7 @@ SIGNATURES = {
     "nva_qk_norm_rope": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i64,
                                    _i32, _i32, _i32, _i32, _f32, _vp]),
     "nva_silu_and_mul": (C.c_int, [_vp, _i64, _vp, _i32, _i32, _vp]),
-    "nva_gather_tokens": (C.c_int, [_vp, _vp, _vp, _i32, _i32, _vp]),
+    "nva_stage_decode_inputs": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _i32, _vp, _i32, _vp]),
     "nva_sample": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _u64, _u64, _vp, _vp, _sz, _i32, _i32, _vp]),
 }
 

@@ -180,7 +180,7 @@ class ModelRunner:
     def _init_decode_staging(self, max_bs: int) -> None:
         """Pinned host buffers and one device buffer holding every per-step decode input; the
         graph's static tensors are typed views into the device buffer, so a decode step needs a
-        single host-to-device copy (the reference issues one copy per tensor plus one device copy
+        single host-to-device transfer (the reference issues one copy per tensor plus one device copy
         per graph variable, nanovllm/engine/model_runner.py:162-179,197-203).  There are two host
         buffers, used in turn: with steps launched ahead of the previous step's tokens the copy
         of one step may still be queued while the host fills in the next."""
@@ -200,6 +200,7 @@ class ModelRunner:
         self._stage_turn = 0
         tdt = {np.int64: torch.int64, np.int32: torch.int32, np.float32: torch.float32}
         self._stage_np, self.graph_vars = [{}, {}], {}
+        self._stage_offsets = {name: off for name, (off, _, _, _) in offsets.items()}
         for name, (off, nbytes, dt, shape) in offsets.items():
             for k in range(2):
                 self._stage_np[k][name] = self._stage_host[k].numpy()[off: off + nbytes].view(dt).reshape(shape)
@@ -228,13 +229,16 @@ class ModelRunner:
         st["context_lens"][bs:bucket] = 0                         # ... and attend over nothing
         st["temperatures"][:bs] = np.fromiter((s.temperature for s in seqs), dtype=np.float32, count=bs)
         st["block_tables"][:bs, : h["block_tables"].shape[1]] = h["block_tables"]   # stale columns stay: never read
-        self._stage_dev.copy_(self._stage_host[self._stage_turn], non_blocking=True)
-        if n_pending:
-            gv = self.graph_vars
-            rc = _lib.load().nva_gather_tokens(gv["input_ids"].data_ptr(), gv["token_src"].data_ptr(),
-                                               prev.tokens_dev.data_ptr(), bs, prev.tokens_dev.numel(),
-                                               torch.cuda.current_stream().cuda_stream)
-            _lib.check(rc, "nva_gather_tokens")
+        # one kernel reads the pinned buffer and writes the device buffer; pending input ids come
+        # from the previous step's sampler output on the way
+        if not n_pending:
+            st["token_src"][:bs] = -1
+        ids_off, idx_off = self._stage_offsets["input_ids"], self._stage_offsets["token_src"]
+        rc = _lib.load().nva_stage_decode_inputs(
+            self._stage_dev.data_ptr(), self._stage_host[self._stage_turn].data_ptr(), self._stage_dev.numel(),
+            ids_off, idx_off, bs, prev.tokens_dev.data_ptr() if n_pending else None,
+            prev.tokens_dev.numel() if n_pending else 0, torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "nva_stage_decode_inputs")
         for graph in self.graphs[bucket]:                         # later segments are enqueued while the first runs
             graph.replay()
         return self.model.compute_logits(self.graph_vars["outputs"][:bs])
