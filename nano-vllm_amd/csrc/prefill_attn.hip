@@ -54,21 +54,34 @@ struct PrefillArgs {
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(const u32x4_t &u) { return __builtin_bit_cast(bf16x8_t, u); }
 
+// max of three in one instruction.  (fmaxf on accumulator registers costs three: the compiler
+// first canonicalises both operands, because it cannot know that they hold no signalling NaN.)
+__device__ __forceinline__ float max3(float x, float y, float z) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
+    return r;
+}
+
 template <bool kPaged>
 __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const PrefillArgs a) {
-    // Workgroups go to the 8 XCDs round-robin by linear id, so the head is the fastest index
-    // (every XCD gets the same mix of tiles however ragged the sequences are) and the query
-    // tiles run from the last one (most keys, longest) to the first.
-    const int h = blockIdx.x % a.num_heads;
-    const int mt = a.num_q_tiles - 1 - (blockIdx.x / a.num_heads) % a.num_q_tiles;
-    const int b = blockIdx.x / (a.num_heads * a.num_q_tiles);
+    // Workgroups go to the 8 XCDs round-robin by linear id and every XCD has an L2 of its own, so
+    // the kv head is the fastest index: with 8 kv heads all workgroups that read the K/V of one
+    // (sequence, kv head) -- every query tile of the query heads sharing it -- run on the same XCD
+    // and find those rows in its L2.  Every XCD still gets the same mix of tiles however ragged
+    // the sequences are.  Query tiles run from the last one (most keys, longest) to the first.
+    const int group = a.num_heads / a.num_kv_heads;
+    const int hkv = blockIdx.x % a.num_kv_heads;
+    int rest = blockIdx.x / a.num_kv_heads;
+    const int h = hkv * group + rest % group;
+    rest /= group;
+    const int mt = a.num_q_tiles - 1 - rest % a.num_q_tiles;
+    const int b = rest / a.num_q_tiles;
     const int q0 = a.cu_seqlens_q[b], k0 = a.cu_seqlens_k[b];
     const int lq = a.cu_seqlens_q[b + 1] - q0;
     const int lk = a.cu_seqlens_k[b + 1] - k0;
     const int row0 = mt * kPfBM;
     if (row0 >= lq) return;                              // also covers empty query spans
     const int off = lk - lq;                             // bottom-right causal alignment
-    const int hkv = h / (a.num_heads / a.num_kv_heads);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -103,51 +116,90 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
 
     // global -> registers for key tile kt: thread t moves chunks t, t+256, t+512, t+768 of the tile
     // (chunk c = key c/16, 16 bytes c%16); keys past the end are clamped and masked later
-    auto load_tile = [&](int kt, u32x4_t (&kr)[4], u32x4_t (&vr)[4]) __attribute__((always_inline)) {
+    // A tile of 64 keys starts at a multiple of 64 and so lies in one 256-token block: its block
+    // id is the same for every lane, and it is fetched one tile ahead of the tile's own loads so
+    // that no load of the loop waits for an address.
+    // (The id is kept in a vector register until it is used: were the compiler to see that it is
+    // uniform it would move it to a scalar register at once, and wait for every load issued before.)
+    int lane_zero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
+    auto fetch_block = [&](int kt) __attribute__((always_inline)) -> int32_t {
+        return kPaged ? a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + ((kt * kPfBN) >> 8) + lane_zero] : 0;
+    };
+    // Addressing: a tile's first row has a wave-uniform address; this lane's chunk of row
+    // tid/16 + 16*r sits a fixed 32-bit byte offset behind it, so a load needs no per-lane 64-bit
+    // arithmetic.  Only the last, partial tile clamps its rows to the last key.
+    const int lkey = tid >> 4, lch = tid & 15;
+    const int64_t kstride = kPaged ? static_cast<int64_t>(a.num_kv_heads) * kHeadDim : a.k_row_stride;
+    const int64_t vstride = kPaged ? kstride : a.v_row_stride;
+    const uint32_t koff0 = static_cast<uint32_t>((lkey * kstride + lch * 8) * 2);
+    const uint32_t voff0 = static_cast<uint32_t>((lkey * vstride + lch * 8) * 2);
+    const uint32_t kstep = static_cast<uint32_t>(16 * kstride * 2), vstep = static_cast<uint32_t>(16 * vstride * 2);
+    auto load_tile = [&](int kt, int32_t blk_v, u32x4_t (&kr)[4], u32x4_t (&vr)[4]) __attribute__((always_inline)) {
+        const int32_t blk = kPaged ? __builtin_amdgcn_readfirstlane(blk_v) : 0;
+        const bool ok = !kPaged || static_cast<uint32_t>(blk) < static_cast<uint32_t>(a.num_blocks);
+        const int key0 = kt * kPfBN;
+        const char *kb, *vb;
+        if (kPaged) {
+            const int64_t e = ((static_cast<int64_t>(ok ? blk : 0) * kBlockSize + (key0 & 255)) * a.num_kv_heads + hkv) *
+                              kHeadDim * 2;
+            kb = reinterpret_cast<const char *>(a.k_cache) + e;
+            vb = reinterpret_cast<const char *>(a.v_cache) + e;
+        } else {
+            kb = reinterpret_cast<const char *>(a.k) + (static_cast<int64_t>(k0 + key0) * kstride + hkv * kHeadDim) * 2;
+            vb = reinterpret_cast<const char *>(a.v) + (static_cast<int64_t>(k0 + key0) * vstride + hkv * kHeadDim) * 2;
+        }
+        if (key0 + kPfBN <= lk) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int c = tid + kPfThreads * r;
-            const int key = c >> 4, ch = c & 15;
-            const int kk = min(kt * kPfBN + key, lk - 1);
-            if (kPaged) {
-                const int32_t blk = a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + (kk >> 8)];
-                if (static_cast<uint32_t>(blk) < static_cast<uint32_t>(a.num_blocks)) {
-                    const int64_t e = ((static_cast<int64_t>(blk) * kBlockSize + (kk & 255)) * a.num_kv_heads + hkv) *
-                                          kHeadDim + ch * 8;
-                    kr[r] = *reinterpret_cast<const u32x4_t *>(a.k_cache + e);
-                    vr[r] = *reinterpret_cast<const u32x4_t *>(a.v_cache + e);
-                } else {
-                    kr[r] = u32x4_t{0u, 0u, 0u, 0u};
-                    vr[r] = u32x4_t{0u, 0u, 0u, 0u};
-                }
-            } else {
-                const int64_t tok = static_cast<int64_t>(k0 + kk);
-                kr[r] = *reinterpret_cast<const u32x4_t *>(a.k + tok * a.k_row_stride + hkv * kHeadDim + ch * 8);
-                vr[r] = *reinterpret_cast<const u32x4_t *>(a.v + tok * a.v_row_stride + hkv * kHeadDim + ch * 8);
+            for (int r = 0; r < 4; ++r) {
+                kr[r] = *reinterpret_cast<const u32x4_t *>(kb + r * kstep + koff0);
+                vr[r] = *reinterpret_cast<const u32x4_t *>(vb + r * vstep + voff0);
+            }
+        } else {
+            const int last = lk - 1 - key0;              // >= 0: rows past it repeat it and are masked later
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = min(lkey + 16 * r, last);
+                kr[r] = *reinterpret_cast<const u32x4_t *>(kb + static_cast<uint32_t>((key * kstride + lch * 8) * 2));
+                vr[r] = *reinterpret_cast<const u32x4_t *>(vb + static_cast<uint32_t>((key * vstride + lch * 8) * 2));
             }
         }
+        return ok;
     };
-    auto store_tile = [&](int buf, const u32x4_t (&kr)[4], const u32x4_t (&vr)[4]) __attribute__((always_inline)) {
+    // registers -> LDS; a tile whose table entry was bad is stored as zeros (its keys then score
+    // 0 and its values add nothing)
+    auto store_tile = [&](int buf, bool ok, const u32x4_t (&kr)[4], const u32x4_t (&vr)[4]) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int c = tid + kPfThreads * r;
             const int key = c >> 4, ch = c & 15;
-            sK[buf][key * 16 + (ch ^ (key & 15))] = kr[r];
-            sV[buf][key * 16 + (ch ^ (4 * (key & 3)))] = vr[r];
+            sK[buf][key * 16 + (ch ^ (key & 15))] = ok ? kr[r] : u32x4_t{0u, 0u, 0u, 0u};
+            sV[buf][key * 16 + (ch ^ (4 * (key & 3)))] = ok ? vr[r] : u32x4_t{0u, 0u, 0u, 0u};
         }
     };
 
     u32x4_t kr[4], vr[4];
-    if (ntiles > 0) {
-        load_tile(0, kr, vr);
-        store_tile(0, kr, vr);
-    }
+    bool tile_ok = true;                                 // of the tile held in kr / vr
+    int32_t blk_next = 0;                                // block id of the tile loaded next
+    if (ntiles > 0) tile_ok = load_tile(0, fetch_block(0), kr, vr);
+    if (ntiles > 1) blk_next = fetch_block(1);
+    // Everything loaded so far (Q above all) is waited for here, and the Q fragments are then
+    // passed through an empty asm.  Without this the compiler keeps treating them as in flight
+    // inside the loop and makes each product wait for the loads issued just before it -- the
+    // next tile's prefetch -- which put a full memory round trip into every tile.
+    __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
+#pragma unroll
+    for (int s = 0; s < 8; ++s) asm volatile("" : "+v"(qfrag[s]));
+    if (ntiles > 0) store_tile(0, tile_ok, kr, vr);
     __syncthreads();
 
     for (int kt = 0; kt < ntiles; ++kt) {
         const int buf = kt & 1;
         const bool more = kt + 1 < ntiles;
-        if (more) load_tile(kt + 1, kr, vr);             // in flight during this tile's arithmetic
+        if (more) {                                      // in flight during this tile's arithmetic
+            tile_ok = load_tile(kt + 1, blk_next, kr, vr);
+            if (kt + 2 < ntiles) blk_next = fetch_block(kt + 2);
+        }
 
         // ---- S^T = K Q^T for two 32-key sub-tiles ----------------------------------------
         f32x16_t sacc[2];
@@ -174,14 +226,19 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
                 for (int i = 0; i < 16; ++i)
                     if (key_base + t2 * 32 + 8 * (i >> 2) + (i & 3) > limit) sacc[t2][i] = -INFINITY;
         }
-        float mloc = fmaxf(sacc[0][0], sacc[1][0]);
+        float mloc0 = max3(sacc[0][0], sacc[0][1], sacc[0][2]), mloc1 = max3(sacc[1][0], sacc[1][1], sacc[1][2]);
+        mloc0 = max3(mloc0, sacc[0][3], sacc[0][4]);
+        mloc1 = max3(mloc1, sacc[1][3], sacc[1][4]);
 #pragma unroll
-        for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(sacc[0][i], sacc[1][i]));
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-        const float m_new = fmaxf(m_run, mloc);
+        for (int i = 5; i < 15; i += 2) {
+            mloc0 = max3(mloc0, sacc[0][i], sacc[0][i + 1]);
+            mloc1 = max3(mloc1, sacc[1][i], sacc[1][i + 1]);
+        }
+        const float mloc = max3(mloc0, mloc1, sacc[0][15] > sacc[1][15] ? sacc[0][15] : sacc[1][15]);
+        const float m_new = max3(m_run, mloc, __shfl_xor(mloc, 32, 64));
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;    // no key seen yet: p = 0
         const float neg_ms = -m_safe * a.scale_log2e;
-        float psum = 0.f;
+        float ps[4] = {0.f, 0.f, 0.f, 0.f};              // four short chains instead of one of 32 adds
         u32x4_t pfrag[2][2];                             // [sub-tile][k-step of 16 keys]
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
@@ -189,7 +246,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 p[i] = __builtin_amdgcn_exp2f(fmaf(sacc[t2][i], a.scale_log2e, neg_ms));   // exp2(-inf) = 0
-                psum += p[i];
+                ps[i & 3] += p[i];
             }
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2)
@@ -205,7 +262,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
                 for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
             m_run = m_new;
         }
-        l_run += psum;
+        l_run += (ps[0] + ps[1]) + (ps[2] + ps[3]);
 
         // ---- O^T += V^T P^T ----------------------------------------------------------------
         // A operand: row = output dim (dt*32 + lane%32), k slot (hh, i) = key 16*s2 + 8*(i/4) + 4*hh + i%4.
@@ -236,7 +293,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
                     }
         }
 
-        if (more) store_tile(buf ^ 1, kr, vr);           // the other buffer was last read before the previous barrier
+        if (more) store_tile(buf ^ 1, tile_ok, kr, vr);           // the other buffer was last read before the previous barrier
         __syncthreads();
     }
 
