@@ -39,6 +39,7 @@ constexpr int kPfThreads = 256;
 constexpr int kPfBM = 128;            // queries per workgroup
 constexpr int kPfBN = 64;             // keys per LDS tile
 constexpr int kPfTileChunks = kPfBN * 16;   // 16-byte chunks per K (or V) tile
+constexpr float kPfLazyLog2 = 8.f;    // how far (in powers of two) the running maximum may run ahead of the exponent base
 
 struct PrefillArgs {
     const bf16_t *q; int64_t q_row_stride;
@@ -216,7 +217,6 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         }
 
         // ---- causal mask, running softmax (base 2; the scale is folded into the exponent) -------
-        // m_run is the running maximum of the RAW scores; p = exp2(scale*log2e * (s - m)).
         const int limit = qrow + off;                    // last key this query may see
         if ((kt * kPfBN + kPfBN - 1) > (wave_qmin + off)) {   // only tiles that cross the diagonal
             const int key_base = kt * kPfBN + 4 * hh;
@@ -235,8 +235,25 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
             mloc1 = max3(mloc1, sacc[1][i], sacc[1][i + 1]);
         }
         const float mloc = max3(mloc0, mloc1, sacc[0][15] > sacc[1][15] ? sacc[0][15] : sacc[1][15]);
-        const float m_new = max3(m_run, mloc, __shfl_xor(mloc, 32, 64));
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;    // no key seen yet: p = 0
+        // m_run is the reference point of the exponentials, p = exp2(scale*log2e * (s - m_run)).  It
+        // follows the true running maximum lazily: only when the maximum has moved more than
+        // kPfLazyLog2 powers of two past it are the sums rescaled (p stays below 2^kPfLazyLog2, far
+        // inside fp32 / bf16 range, and the final division by the row sum cancels the common
+        // factor exactly).  With an eager update nearly every tile of a short sequence moves the
+        // maximum of some query of the wavefront, and every move costs 64 multiplications per lane.
+        const float m_true = max3(m_run, mloc, __shfl_xor(mloc, 32, 64));
+        const bool lift = (m_true - m_run) * a.scale_log2e > kPfLazyLog2;   // -inf - -inf = NaN: false
+        if (__builtin_amdgcn_ballot_w64(lift) != 0) {
+            const float m_to = lift ? m_true : m_run;
+            const float alpha = lift ? __builtin_amdgcn_exp2f((m_run - m_to) * a.scale_log2e) : 1.f;   // 0 on first use
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+            m_run = m_to;
+        }
+        const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;    // no key seen yet: p = 0
         const float neg_ms = -m_safe * a.scale_log2e;
         float ps[4] = {0.f, 0.f, 0.f, 0.f};              // four short chains instead of one of 32 adds
         u32x4_t pfrag[2][2];                             // [sub-tile][k-step of 16 keys]
@@ -252,15 +269,6 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
             for (int s2 = 0; s2 < 2; ++s2)
                 pfrag[t2][s2] = u32x4_t{pack_bf16x2(p[8 * s2 + 0], p[8 * s2 + 1]), pack_bf16x2(p[8 * s2 + 2], p[8 * s2 + 3]),
                                         pack_bf16x2(p[8 * s2 + 4], p[8 * s2 + 5]), pack_bf16x2(p[8 * s2 + 6], p[8 * s2 + 7])};
-        }
-        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {     // some query of the wavefront moved its maximum
-            const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * a.scale_log2e);   // exp2(-inf) = 0 on first use
-            l_run *= alpha;
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-            m_run = m_new;
         }
         l_run += (ps[0] + ps[1]) + (ps[2] + ps[3]);
 
