@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
 
 A "step" is one pass of the selected workload over one batch of synthetic input that is
-already resident in HBM.  Workloads (shapes are the BASELINE.json configs):
+already resident in HBM.  Workloads (shapes are the five benchmark configurations):
     e2e       (default) generate() over 256 requests on a Qwen3-0.6B-architecture model (config 4)
     longctx   Qwen3-8B-architecture long-context decode stress, batch 128, ctx U[4096,16384]  (config 5)
     decode    paged decode attention, batch 64, 16/8 heads, ctx U[100,2048]       (config 2)

@@ -20,9 +20,12 @@ constexpr int kNormMaxChunks = 8;     // 8 x (64 lanes x 8 elements) = hidden si
 
 __device__ __forceinline__ float round_bf16(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 
-// One wavefront per row, the row lives in registers between the two passes.
-// residual == nullptr: out = bf16(x * rsqrt(mean(x^2) + eps)) * w
-// else:                s = x + residual (fp32); residual_out = bf16(s); out = bf16(s * rsqrt(mean(s^2) + eps)) * w
+// One wavefront per row, the row lives in registers between the two passes.  NC = chunks of 512
+// elements per row; every load of the row (input, residual and weight) is issued before the first
+// use, so the kernel costs one memory round trip instead of one per chunk and tensor.
+// kResidual false: out = bf16(x * rsqrt(mean(x^2) + eps)) * w
+// else:            s = x + residual (fp32); residual_out = bf16(s); out = bf16(s * rsqrt(mean(s^2) + eps)) * w
+template <int NC, bool kResidual>
 __global__ __launch_bounds__(256) void rms_norm_kernel(
     const bf16_t *__restrict__ x, int64_t x_stride, const bf16_t *__restrict__ residual, int64_t res_stride,
     const bf16_t *__restrict__ weight, bf16_t *__restrict__ out, bf16_t *__restrict__ residual_out,
@@ -31,26 +34,34 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
     const bf16_t *xr = x + static_cast<int64_t>(row) * x_stride;
-    const bf16_t *rr = residual ? residual + static_cast<int64_t>(row) * res_stride : nullptr;
-    float v[kNormMaxChunks][8];
+    const bf16_t *rr = kResidual ? residual + static_cast<int64_t>(row) * res_stride : nullptr;
+    uint4 xv[NC], rv[NC], wv[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int e = min(c * 512 + lane * 8, hidden - 8);       // lanes past the row re-read its end
+        xv[c] = *reinterpret_cast<const uint4 *>(xr + e);
+        if (kResidual) rv[c] = *reinterpret_cast<const uint4 *>(rr + e);
+        wv[c] = *reinterpret_cast<const uint4 *>(weight + e);
+    }
+    float v[NC][8];
     float ss = 0.f;
 #pragma unroll
-    for (int c = 0; c < kNormMaxChunks; ++c) {
-        const int e = c * 512 + lane * 8;
-        if (e < hidden) {
-            const uint4 xv = *reinterpret_cast<const uint4 *>(xr + e);
-            unpack8(xv, v[c]);
-            if (rr) {
-                const uint4 rv = *reinterpret_cast<const uint4 *>(rr + e);
-                float rf[8];
-                unpack8(rv, rf);
+    for (int c = 0; c < NC; ++c) {
+        const bool live = c * 512 + lane * 8 < hidden;
+        unpack8(xv[c], v[c]);
+        if (kResidual) {
+            float rf[8];
+            unpack8(rv[c], rf);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[c][i] += rf[i];
+            for (int i = 0; i < 8; ++i) v[c][i] += rf[i];
+            if (live) {
                 uint4 ro;
                 ro.x = pack_bf16x2(v[c][0], v[c][1]); ro.y = pack_bf16x2(v[c][2], v[c][3]);
                 ro.z = pack_bf16x2(v[c][4], v[c][5]); ro.w = pack_bf16x2(v[c][6], v[c][7]);
-                *reinterpret_cast<uint4 *>(residual_out + static_cast<int64_t>(row) * hidden + e) = ro;
+                *reinterpret_cast<uint4 *>(residual_out + static_cast<int64_t>(row) * hidden + c * 512 + lane * 8) = ro;
             }
+        }
+        if (live) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) ss = fmaf(v[c][i], v[c][i], ss);
         }
@@ -58,20 +69,31 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
     ss = wave_sum(ss);
     const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
 #pragma unroll
-    for (int c = 0; c < kNormMaxChunks; ++c) {
-        const int e = c * 512 + lane * 8;
-        if (e < hidden) {
-            const uint4 wv = *reinterpret_cast<const uint4 *>(weight + e);
+    for (int c = 0; c < NC; ++c) {
+        if (c * 512 + lane * 8 < hidden) {
             float wf[8], y[8];
-            unpack8(wv, wf);
+            unpack8(wv[c], wf);
 #pragma unroll
             for (int i = 0; i < 8; ++i) y[i] = round_bf16(v[c][i] * inv) * wf[i];
             uint4 o;
             o.x = pack_bf16x2(y[0], y[1]); o.y = pack_bf16x2(y[2], y[3]);
             o.z = pack_bf16x2(y[4], y[5]); o.w = pack_bf16x2(y[6], y[7]);
-            *reinterpret_cast<uint4 *>(out + static_cast<int64_t>(row) * hidden + e) = o;
+            *reinterpret_cast<uint4 *>(out + static_cast<int64_t>(row) * hidden + c * 512 + lane * 8) = o;
         }
     }
+}
+
+template <int NC>
+static void launch_rms_norm(hipStream_t stream, const bf16_t *x, int64_t x_stride, const bf16_t *residual,
+                            int64_t res_stride, const bf16_t *weight, bf16_t *out, bf16_t *residual_out,
+                            int32_t rows, int32_t hidden, float eps) {
+    const dim3 grid((rows + 3) / 4), block(256);
+    if (residual)
+        hipLaunchKernelGGL((rms_norm_kernel<NC, true>), grid, block, 0, stream, x, x_stride, residual, res_stride, weight,
+                           out, residual_out, rows, hidden, eps);
+    else
+        hipLaunchKernelGGL((rms_norm_kernel<NC, false>), grid, block, 0, stream, x, x_stride, residual, res_stride, weight,
+                           out, residual_out, rows, hidden, eps);
 }
 
 // One wavefront per (token, head) row of 128 elements; lane l holds elements l and l + 64,
@@ -191,10 +213,20 @@ extern "C" int nva_rms_norm(const void *x, int64_t x_row_stride, const void *res
     if (residual && (residual_row_stride < hidden || residual_row_stride % 8 != 0)) return NVA_ERR_BAD_STRIDE;
     if (!aligned16(x) || !aligned16(weight) || !aligned16(out) || (residual && (!aligned16(residual) || !aligned16(residual_out))))
         return NVA_ERR_MISALIGNED;
-    hipLaunchKernelGGL(rms_norm_kernel, dim3((rows + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const bf16_t *>(x), x_row_stride, static_cast<const bf16_t *>(residual),
-                       residual_row_stride, static_cast<const bf16_t *>(weight), static_cast<bf16_t *>(out),
-                       static_cast<bf16_t *>(residual_out), rows, hidden, eps);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bf16_t *xp = static_cast<const bf16_t *>(x), *rp = static_cast<const bf16_t *>(residual);
+    const bf16_t *wp = static_cast<const bf16_t *>(weight);
+    bf16_t *op = static_cast<bf16_t *>(out), *rop = static_cast<bf16_t *>(residual_out);
+    switch ((hidden + 511) / 512) {
+        case 1: launch_rms_norm<1>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
+        case 2: launch_rms_norm<2>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
+        case 3: launch_rms_norm<3>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
+        case 4: launch_rms_norm<4>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
+        case 5: launch_rms_norm<5>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
+        case 6: launch_rms_norm<6>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
+        case 7: launch_rms_norm<7>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
+        default: launch_rms_norm<8>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
+    }
     return launch_status();
 }
 

@@ -49,7 +49,7 @@ def test_model_steps_match_cpu_oracle_model(runner):
         return s
 
     first = mk(300, [5, 9])
-    # round 1: fills blocks 5 and 9 (block 5 becomes a reusable full prefix block)
+    # first pass: fills blocks 5 and 9 (block 5 becomes a reusable full prefix block)
     for seqs in ([first], [mk(700, [1, 2, 3]), mk(290, [5, 11], cached=256, ids=first.token_ids[:256] + [7] * 34), mk(33, [20])]):
         h = build_prefill_inputs(seqs, 256)
         ids, pos = runner.prepare_prefill(seqs)
