@@ -202,6 +202,9 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
             if (kt + 2 < ntiles) blk_next = fetch_block(kt + 2);
         }
 
+        // A wavefront skips the arithmetic of a tile that lies wholly beyond the diagonal for all
+        // of its 32 queries (the tile exists because later wavefronts of the workgroup see it).
+        if (kt * kPfBN <= wave_qmin + 31 + off) {
         // ---- S^T = K Q^T for two 32-key sub-tiles ----------------------------------------
         f32x16_t sacc[2];
 #pragma unroll
@@ -301,6 +304,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
                     }
         }
 
+        }
         if (more) store_tile(buf ^ 1, tile_ok, kr, vr);           // the other buffer was last read before the previous barrier
         __syncthreads();
     }
