@@ -202,7 +202,7 @@ def bench_sampler(args, dev):
                    "batch": batch},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "sampler_partials_kernel + sampler_argmax_kernel + sampler_pick_kernel",
+                     "kernel": "sampler_gumbel_kernel + sampler_pick_kernel",
                      "algorithmic_bytes_per_launch": alg},
     }
 
@@ -235,22 +235,20 @@ def e2e_workload(num_seqs=256, max_input_len=1024, max_output_len=1024, vocab=15
 MEASURED_TRAFFIC_E2E_SHAPE = 874_900_000      # stream kernel 869.9 MB + merge kernel 5.0 MB (algorithmic: 855.3 MB)
 
 
-def decode_e2e_shape_roofline(dev, caches, num_blocks):
-    """Paged decode attention at the e2e workload's own decode shape: the 256 requests of the bench
-    mix mid-flight (context = prompt + half of the output, mean 813 tokens), block tables drawn
-    without replacement from the pool, timed with HIP events while rotating through `caches`
-    (separate K/V pools, so neither L2 nor the 256 MB Infinity Cache can serve re-reads)."""
+def decode_shape_roofline(dev, caches, num_blocks, ctx, hq, what, traffic=None, width=None):
+    """Paged decode attention for the context lengths ``ctx``: block tables drawn without
+    replacement from the pool, timed with HIP events while rotating through `caches` (separate
+    K/V pools, so neither L2 nor the 256 MB Infinity Cache can serve re-reads)."""
     import torch
     import nanovllm_amd as nva
     from nanovllm_amd import synthetic
-    prompts, params = e2e_workload()
     g = torch.Generator().manual_seed(1)
-    ctx = torch.tensor([len(p) + sp.max_tokens // 2 for p, sp in zip(prompts, params)], dtype=torch.int32)
-    tables = synthetic.decode_tables(ctx.tolist(), num_blocks, g, width=16).to(dev)
+    batch = ctx.numel()
+    tables = synthetic.decode_tables(ctx.tolist(), num_blocks, g, width=width).to(dev)
     ctx_d = ctx.to(dev)
-    hq, hkv, dh = 16, caches[0][0].shape[2], caches[0][0].shape[3]
-    q = torch.randn(256, hq, dh, device=dev).to(torch.bfloat16)
-    out = torch.empty(256, 1, hq, dh, dtype=torch.bfloat16, device=dev)
+    hkv, dh = caches[0][0].shape[2], caches[0][0].shape[3]
+    q = torch.randn(batch, hq, dh, device=dev).to(torch.bfloat16)
+    out = torch.empty(batch, 1, hq, dh, dtype=torch.bfloat16, device=dev)
     scale = dh ** -0.5
     fns = [lambda kc=kc, vc=vc: nva.paged_decode_attention(q, kc, vc, ctx_d, tables, scale, out=out)
            for kc, vc in caches]
@@ -259,10 +257,41 @@ def decode_e2e_shape_roofline(dev, caches, num_blocks):
     alg = int(ctx.sum()) * hkv * dh * 2 * 2 + 2 * q.numel() * 2
     gbps = alg / (ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_E2E_SHAPE,
-            "kernel": "decode_stream_kernel<2> (+ decode_merge_kernel<2>): paged decode attention, batch 256, "
-                      "mean ctx %d" % int(ctx.float().mean()),
+            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
+            "kernel": "decode_stream_kernel<%d> (+ decode_merge_kernel<%d>): paged decode attention, %s, mean ctx %d"
+                      % (hq // hkv, hq // hkv, what, int(ctx.float().mean())),
             "algorithmic_bytes_per_launch": alg, "us_per_launch": round(ms * 1e3, 2)}
+
+
+def decode_e2e_shape_roofline(dev, caches, num_blocks):
+    """The e2e workload's own decode shape: the 256 requests of the bench mix mid-flight (context =
+    prompt + half of the output, mean 813 tokens)."""
+    import torch
+    prompts, params = e2e_workload()
+    ctx = torch.tensor([len(p) + sp.max_tokens // 2 for p, sp in zip(prompts, params)], dtype=torch.int32)
+    return decode_shape_roofline(dev, caches, num_blocks, ctx, 16, "batch 256", MEASURED_TRAFFIC_E2E_SHAPE,
+                                 width=16)           # the engine's static table width at max_model_len 4096
+
+
+def bench_decode_longctx_shape(args, dev):
+    """One layer of the long-context stress (config 5): batch 128, contexts U[4096,16384], 32 query
+    / 8 kv heads; 4 private pools sized to the drawn contexts (about 5300 blocks, 2.8 GB each for K and for V)."""
+    import random
+    import torch
+    rng = random.Random(0)
+    ctx = torch.tensor([rng.randint(4096, 16384) for _ in range(128)], dtype=torch.int32)
+    need = int(((ctx + 255) // 256).sum())
+    caches = []
+    for p in range(4):
+        g = torch.Generator(device=dev).manual_seed(300 + p)
+        caches.append(tuple(torch.empty((need + 8, 256, 8, 128), device=dev, dtype=torch.bfloat16).normal_(generator=g)
+                            for _ in range(2)))
+    roof = decode_shape_roofline(dev, caches, need + 8, ctx, 32, "batch 128, ctx U[4096,16384]")
+    result = {"metric": "paged decode attention at the long-context shape (config 5, one layer), achieved HBM GB/s",
+              "value": roof["achieved"], "unit": "GB/s", "ms_per_step": round(roof["us_per_launch"] / 1e3, 5),
+              "config": {"workload": "paged_decode_attn, batch 128, 32q/8kv heads, contexts U[4096,16384], "
+                                     "4 rotating pools of %d blocks" % (need + 8)}, "roofline": roof}
+    return result, (lambda: None)
 
 
 def bench_decode_e2e_shape(args, dev):
@@ -423,8 +452,9 @@ def bench_longctx(args, dev):
     return result, (lambda: None)
 
 
-WORKLOADS = {"e2e": bench_e2e, "longctx": bench_longctx, "decode-e2e-shape": bench_decode_e2e_shape, "copy": bench_copy, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
-DEFAULT_STEPS = {"e2e": 1, "longctx": 1, "decode-e2e-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
+WORKLOADS = {"e2e": bench_e2e, "longctx": bench_longctx, "decode-e2e-shape": bench_decode_e2e_shape,
+             "decode-longctx-shape": bench_decode_longctx_shape, "copy": bench_copy, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
+DEFAULT_STEPS = {"e2e": 1, "longctx": 1, "decode-e2e-shape": 1, "decode-longctx-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
 
 
 def main():
