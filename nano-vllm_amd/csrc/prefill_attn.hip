@@ -125,7 +125,8 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     int lane_zero;
     asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
     auto fetch_block = [&](int kt) __attribute__((always_inline)) -> int32_t {
-        return kPaged ? a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + ((kt * kPfBN) >> 8) + lane_zero] : 0;
+        // (the column is clamped to the row: cu_seqlens_k is device data the host could not check)
+        return kPaged ? a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + min((kt * kPfBN) >> 8, a.bt_row_stride - 1) + lane_zero] : 0;
     };
     // Addressing: a tile's first row has a wave-uniform address; this lane's chunk of row
     // tid/16 + 16*r sits a fixed 32-bit byte offset behind it, so a load needs no per-lane 64-bit
