@@ -132,6 +132,21 @@ def test_sampler_validation_and_workspace_size():
     assert f(A, 100, A, None, 0, 0, 0, A, A, 1 << 20, 0, 100, None) == _lib.OK
 
 
+def test_stage_decode_inputs_validation():
+    f = _lib.load().nva_stage_decode_inputs
+    # (dst, src_host, nbytes, ids_offset, index_offset, n, prev_tokens, n_prev, stream)
+    assert f(None, A, 4096, 0, 2048, 16, None, 0, None) == _lib.ERR_NULL_POINTER
+    assert f(A, A, 4096, 0, 2048, 16, None, 4, None) == _lib.ERR_NULL_POINTER               # tokens announced, none given
+    assert f(A, A, 4100, 0, 2048, 16, None, 0, None) == _lib.ERR_MISALIGNED                 # whole 16-byte chunks only
+    assert f(A, A, 4096, 8, 2048, 16, None, 0, None) == _lib.ERR_MISALIGNED
+    assert f(A + 8, A, 4096, 0, 2048, 16, None, 0, None) == _lib.ERR_MISALIGNED
+    assert f(A, A, 4096, 0, 2048, 1024, None, 0, None) == _lib.ERR_BAD_SHAPE                # ids run past the buffer
+    assert f(A, A, 4096, 0, 4090, 16, None, 0, None) == _lib.ERR_MISALIGNED
+    assert f(A, A, 4096, 0, 4092, 16, None, 0, None) == _lib.ERR_BAD_SHAPE                  # index runs past the buffer
+    assert f(A, A, -16, 0, 0, 0, None, 0, None) == _lib.ERR_BAD_SHAPE
+    assert f(None, None, 0, 0, 0, 0, None, 0, None) == _lib.OK                              # nothing to move
+
+
 def test_python_wrappers_refuse_cpu_tensors_and_keep_reference_asserts():
     import nanovllm_amd as nva
     k = torch.zeros(4, 8, 128, dtype=torch.bfloat16)

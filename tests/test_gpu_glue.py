@@ -100,3 +100,35 @@ def test_qk_norm_rope_fused_scatter_matches_store_kvcache(dev):
     torch.cuda.synchronize()
     assert torch.equal(q1, q2) and torch.equal(k1, k2)
     assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2) and bool(kc1.any()) and bool(vc1.any())
+
+
+@pytest.mark.gpu
+def test_stage_decode_inputs_copies_and_hands_over_tokens(dev):
+    """The staging kernel copies the pinned buffer bit for bit and replaces exactly the input
+    ids whose index names a row of the previous step's tokens (-1 and out-of-range keep the
+    host's value)."""
+    from nanovllm_amd import _lib
+    lib = _lib.load()
+    n, n_prev, nbytes = 37, 19, 4096
+    ids_off, idx_off = 256, 1024                                    # int64 ids, int32 indices inside the buffer
+    host = torch.randint(0, 255, (nbytes,), dtype=torch.uint8).pin_memory()
+    ids = host[ids_off: ids_off + 8 * n].view(torch.int64)
+    idx = host[idx_off: idx_off + 4 * n].view(torch.int32)
+    g = torch.Generator().manual_seed(0)
+    ids.copy_(torch.randint(0, 150000, (n,), generator=g))
+    idx.copy_(torch.randint(-1, n_prev + 3, (n,), generator=g, dtype=torch.int32))   # includes -1 and too large
+    prev = torch.randint(0, 150000, (n_prev,), generator=g).to(dev)
+    dst = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    rc = lib.nva_stage_decode_inputs(dst.data_ptr(), host.data_ptr(), nbytes, ids_off, idx_off, n, prev.data_ptr(),
+                                     n_prev, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    want = host.clone()
+    want_ids = want[ids_off: ids_off + 8 * n].view(torch.int64)
+    take = (idx >= 0) & (idx < n_prev)
+    want_ids[take] = prev.cpu()[idx[take].long()]
+    assert torch.equal(dst.cpu(), want)
+    assert take.any() and (~take).any()
+    # without previous tokens it is a plain copy
+    rc = lib.nva_stage_decode_inputs(dst.data_ptr(), host.data_ptr(), nbytes, ids_off, idx_off, n, None, 0,
+                                     torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and torch.equal(dst.cpu(), host)
