@@ -136,3 +136,47 @@ def test_decode_partials_are_fresh_across_calls(dev):
         i = it & 1
         out = paged_decode_attention(*dev_in[i], cases[i].scale)
         assert torch.equal(out, good[i]), f"iteration {it}"
+
+
+def test_decode_config5_full_size(dev):
+    """The long-context stress shape at full size: batch 128, 32 q / 8 kv heads, contexts
+    U[4096,16384], blocks scattered over a 5.4 GB pool.  Too big for the oracle as a whole, so:
+    three sequences are re-stated as a small case (their pages gathered, tables renumbered) and
+    checked against the fp32 oracle, both as rows of the big launch and launched alone (a
+    different split of the work); the output does not depend on the physical placement of the
+    blocks (bit for bit); V == 1 gives 1."""
+    g = torch.Generator().manual_seed(5)
+    ctx = torch.randint(4096, 16385, (128,), generator=g, dtype=torch.int32)
+    need = int(((ctx + 255) // 256).sum())
+    tables = synthetic.decode_tables(ctx.tolist(), need + 8, g)
+    gd = torch.Generator(device=dev).manual_seed(6)
+    kc = torch.empty((need + 8, 256, 8, 128), device=dev, dtype=torch.bfloat16).normal_(generator=gd)
+    vc = torch.empty((need + 8, 256, 8, 128), device=dev, dtype=torch.bfloat16).normal_(generator=gd)
+    q = torch.randn((128, 32, 128), generator=g).to(torch.bfloat16)
+    scale = 128 ** -0.5
+    out = paged_decode_attention(q.to(dev), kc, vc, ctx.to(dev), tables.to(dev), scale)
+    torch.cuda.synchronize()
+    assert out.shape == (128, 1, 32, 128)
+    pick = [0, 57, 127, int(ctx.argmax()), int(ctx.argmin())]
+    # the picked sequences as a case of their own: pages gathered to a private pool
+    blocks = [tables[b, : (int(ctx[b]) + 255) // 256].long() for b in pick]
+    flat = torch.cat(blocks)
+    small_k, small_v = kc[flat.to(dev)].cpu(), vc[flat.to(dev)].cpu()
+    small_t = torch.full((len(pick), tables.shape[1]), -1, dtype=torch.int32)
+    at = 0
+    for i, blk in enumerate(blocks):
+        small_t[i, : len(blk)] = torch.arange(at, at + len(blk), dtype=torch.int32)
+        at += len(blk)
+    want = oracle.paged_decode_attention(q[pick], small_k, small_v, ctx[pick], small_t, scale, "fp32")
+    assert_attn_close(out[pick], want, "config 5 rows vs oracle")
+    alone = paged_decode_attention(q[pick].to(dev), small_k.to(dev), small_v.to(dev), ctx[pick].to(dev),
+                                   small_t.to(dev), scale)
+    assert_attn_close(alone, want, "config 5 rows alone")
+    # physical placement: reverse the pool
+    rev = torch.arange(need + 7, -1, -1)
+    t2 = torch.where(tables >= 0, (need + 7 - tables.clamp_min(0)).to(torch.int32), tables)
+    out2 = paged_decode_attention(q.to(dev), kc[rev.to(dev)], vc[rev.to(dev)], ctx.to(dev), t2.to(dev), scale)
+    assert torch.equal(bits(out2), bits(out))
+    del out2
+    ones = paged_decode_attention(q.to(dev), kc, torch.ones_like(vc), ctx.to(dev), tables.to(dev), scale)
+    assert (ones.float() - 1).abs().max().item() < 1e-2

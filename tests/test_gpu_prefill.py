@@ -118,3 +118,28 @@ def test_prefill_sequences_do_not_leak(dev):
     out2, _ = _packed(case2, dev)
     assert torch.equal(bits(out[:a]), bits(out2[:a])) and torch.equal(bits(out[b:]), bits(out2[b:]))
     assert not torch.equal(bits(out[a:b]), bits(out2[a:b]))
+
+
+def test_prefill_warmup_shape_4x4096(dev):
+    """The runner's warm-up batch (4 sequences of max_model_len = 4096 tokens, packed, no cache):
+    64 key tiles per row, far more than config 3 has.  One sequence is checked against the fp32
+    oracle in full; every sequence launched alone gives the same bits as inside the batch."""
+    g = torch.Generator().manual_seed(21)
+    n, L = 4, 4096
+    q = (torch.randn((n * L, 16, 128), generator=g)).to(torch.bfloat16)
+    k = (torch.randn((n * L, 8, 128), generator=g)).to(torch.bfloat16)
+    v = (torch.randn((n * L, 8, 128), generator=g)).to(torch.bfloat16)
+    cu = torch.arange(0, (n + 1) * L, L, dtype=torch.int32)
+    scale = 128 ** -0.5
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out = varlen_prefill_attention(qd, kd, vd, cu.to(dev), cu.to(dev), L, L, scale)
+    torch.cuda.synchronize()
+    one = torch.tensor([0, L], dtype=torch.int32)
+    s = 2                                                        # the sequence given to the oracle
+    want = oracle.varlen_prefill_attention(q[s * L:(s + 1) * L], k[s * L:(s + 1) * L], v[s * L:(s + 1) * L], one, one,
+                                           scale, precision="fp32")
+    assert_attn_close(out[s * L:(s + 1) * L], want, "4096-token sequence")
+    for i in range(n):
+        alone = varlen_prefill_attention(qd[i * L:(i + 1) * L], kd[i * L:(i + 1) * L], vd[i * L:(i + 1) * L],
+                                         one.to(dev), one.to(dev), L, L, scale)
+        assert torch.equal(bits(alone), bits(out[i * L:(i + 1) * L]))
