@@ -232,7 +232,7 @@ def e2e_workload(num_seqs=256, max_input_len=1024, max_output_len=1024, vocab=15
 # HBM bytes per launch of decode_stream_kernel<2> at the e2e decode shape, from two rocprofv3 --pmc
 # passes of `bench.py --workload decode-e2e-shape` (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each
 # scaled by what the same counter reads for the plain copy kernel of `--workload copy` (known size).
-MEASURED_TRAFFIC_E2E_SHAPE = 874_900_000      # stream kernel 869.9 MB + merge kernel 5.0 MB (algorithmic: 855.3 MB)
+MEASURED_TRAFFIC_E2E_SHAPE = 863_700_000      # stream kernel 858.8 MB + merge kernel 4.9 MB (algorithmic: 855.3 MB)
 
 
 def decode_shape_roofline(dev, caches, num_blocks, ctx, hq, what, traffic=None, width=None):
