@@ -235,10 +235,12 @@ def e2e_workload(num_seqs=256, max_input_len=1024, max_output_len=1024, vocab=15
 MEASURED_TRAFFIC_E2E_SHAPE = 863_700_000      # stream kernel 858.8 MB + merge kernel 4.9 MB (algorithmic: 855.3 MB)
 
 
-def decode_shape_roofline(dev, caches, num_blocks, ctx, hq, what, traffic=None, width=None):
+def decode_shape_roofline(dev, caches, num_blocks, ctx, hq, what, traffic=None, width=None, layers=None):
     """Paged decode attention for the context lengths ``ctx``: block tables drawn without
     replacement from the pool, timed with HIP events while rotating through `caches` (separate
-    K/V pools, so neither L2 nor the 256 MB Infinity Cache can serve re-reads)."""
+    K/V pools, so neither L2 nor the 256 MB Infinity Cache can serve re-reads).  With ``layers``
+    the calls are grouped as the engine groups them: every ``layers`` consecutive calls share
+    one work split, derived by the first of them (the layers of one decode step)."""
     import torch
     import nanovllm_amd as nva
     from nanovllm_amd import synthetic
@@ -250,16 +252,26 @@ def decode_shape_roofline(dev, caches, num_blocks, ctx, hq, what, traffic=None, 
     q = torch.randn(batch, hq, dh, device=dev).to(torch.bfloat16)
     out = torch.empty(batch, 1, hq, dh, dtype=torch.bfloat16, device=dev)
     scale = dh ** -0.5
-    fns = [lambda kc=kc, vc=vc: nva.paged_decode_attention(q, kc, vc, ctx_d, tables, scale, out=out)
-           for kc, vc in caches]
-    reps = max(5 * len(fns), 60)
-    ms = _event_time_ms(fns, reps, len(fns)) / reps
+    from nanovllm_amd.context import DecodePlan
+    state = {"calls": 0, "plan": None}
+
+    def call(kc, vc):
+        if layers:
+            if state["calls"] % layers == 0:
+                state["plan"] = DecodePlan()
+            state["calls"] += 1
+        nva.paged_decode_attention(q, kc, vc, ctx_d, tables, scale, out=out, plan=state["plan"])
+
+    fns = [lambda kc=kc, vc=vc: call(kc, vc) for kc, vc in caches]
+    reps = 3 * layers if layers else max(5 * len(fns), 60)      # whole steps: one build per `layers` calls
+    ms = _event_time_ms(fns, reps, layers if layers else len(fns)) / reps
     alg = int(ctx.sum()) * hkv * dh * 2 * 2 + 2 * q.numel() * 2
     gbps = alg / (ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
-            "kernel": "decode_stream_kernel<%d> (+ decode_merge_kernel<%d>): paged decode attention, %s, mean ctx %d"
-                      % (hq // hkv, hq // hkv, what, int(ctx.float().mean())),
+            "kernel": "decode_stream_kernel<%d> (+ decode_merge_kernel<%d>): paged decode attention, %s, mean ctx %d%s"
+                      % (hq // hkv, hq // hkv, what, int(ctx.float().mean()),
+                         ", %d layers per work split" % layers if layers else ""),
             "algorithmic_bytes_per_launch": alg, "us_per_launch": round(ms * 1e3, 2)}
 
 
@@ -270,7 +282,8 @@ def decode_e2e_shape_roofline(dev, caches, num_blocks):
     prompts, params = e2e_workload()
     ctx = torch.tensor([len(p) + sp.max_tokens // 2 for p, sp in zip(prompts, params)], dtype=torch.int32)
     return decode_shape_roofline(dev, caches, num_blocks, ctx, 16, "batch 256", MEASURED_TRAFFIC_E2E_SHAPE,
-                                 width=16)           # the engine's static table width at max_model_len 4096
+                                 width=16,           # the engine's static table width at max_model_len 4096
+                                 layers=28)          # Qwen3-0.6B
 
 
 def bench_decode_longctx_shape(args, dev):
@@ -286,7 +299,7 @@ def bench_decode_longctx_shape(args, dev):
         g = torch.Generator(device=dev).manual_seed(300 + p)
         caches.append(tuple(torch.empty((need + 8, 256, 8, 128), device=dev, dtype=torch.bfloat16).normal_(generator=g)
                             for _ in range(2)))
-    roof = decode_shape_roofline(dev, caches, need + 8, ctx, 32, "batch 128, ctx U[4096,16384]")
+    roof = decode_shape_roofline(dev, caches, need + 8, ctx, 32, "batch 128, ctx U[4096,16384]", layers=36)
     result = {"metric": "paged decode attention at the long-context shape (config 5, one layer), achieved HBM GB/s",
               "value": roof["achieved"], "unit": "GB/s", "ms_per_step": round(roof["us_per_launch"] / 1e3, 5),
               "config": {"workload": "paged_decode_attn, batch 128, 32q/8kv heads, contexts U[4096,16384], "

@@ -94,6 +94,31 @@ int nva_paged_decode_attn(const void *q, int64_t q_row_stride,
                           float scale, void *stream);
 
 /*
+ * The same operation for a caller that makes several calls over the SAME context_lens and
+ * block_tables contents, batch, head counts and workspace, ordered on one stream -- the
+ * layers of one decode step (the loop over decoder layers around
+ * nanovllm/layers/attention.py:71-74 changes only q and the cache pointers).
+ *   plan == NVA_PLAN_BUILD: as nva_paged_decode_attn; the work split it derives from
+ *     context_lens and block_tables stays in the workspace.
+ *   plan == NVA_PLAN_REUSE: takes the split the last NVA_PLAN_BUILD call left in this
+ *     workspace instead of deriving it again (saves a few microseconds per launch).  The caller
+ *     guarantees that call had the same batch, head counts, num_blocks and table contents
+ *     and that nothing else wrote the workspace since; otherwise the result is undefined
+ *     (memory accesses stay inside the caches as long as the old block numbers were valid).
+ * Batches above 1024 sequences are run as several launches and always rebuild.
+ */
+enum { NVA_PLAN_BUILD = 0, NVA_PLAN_REUSE = 1 };
+
+int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride,
+                                  const void *k_cache, const void *v_cache,
+                                  const int32_t *block_tables, int32_t bt_row_stride,
+                                  int32_t max_blocks, const int32_t *context_lens,
+                                  void *out, void *workspace, size_t workspace_bytes,
+                                  int32_t batch, int32_t num_heads, int32_t num_kv_heads,
+                                  int32_t head_dim, int32_t block_size, int32_t num_blocks,
+                                  float scale, int32_t plan, void *stream);
+
+/*
  * Causal variable-length prefill attention, optionally reading K/V through the paged
  * cache.  Replaces the flash_attn_varlen_func call of Attention.forward
  * (nanovllm/layers/attention.py:64-70).

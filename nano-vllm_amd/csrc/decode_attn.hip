@@ -75,13 +75,19 @@ struct DecodeArgs {
     const int32_t *context_lens;
     bf16_t *out;
     int32_t *pref_out;       // [batch + 1] stage-count prefix sums, written for the merge kernel
+    int32_t *ctx_out;        // [batch] clipped context lengths       } the work split, kept for later
+    int32_t *rec_out;        // [kDecWorkers][8] first stage per worker } launches over the same contexts
     float *part_ml;          // [rows][2]
     float *part_o;           // [rows][128]
     int32_t batch, max_blocks, num_heads, num_kv_heads, num_blocks;
     float scale_log2e;
 };
 
-template <int G>
+// kReuse: the workspace already holds the work split of an earlier launch (kReuse = false) over
+// the same context_lens and block_tables; each worker then starts from its 32-byte record and
+// issues its first loads before anything else, instead of prefix-summing the context lengths and
+// reading the block table first.
+template <int G, bool kReuse>
 __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const DecodeArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -93,87 +99,24 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
     __shared__ int32_t sh_pref[kDecMaxBatch + 1];   // sh_pref[b] = stages of all (sequence < b, head)
     __shared__ int32_t sh_ctx[kDecMaxBatch];        // context length of sequence b, clipped to the table
     __shared__ __attribute__((aligned(16))) u32x4_t lds[kDecWaves * kWaveLdsChunks];
-    if (wave == 0) {
-        constexpr int kPer = kDecMaxBatch / kWave;  // 16 sequences per lane
-        int cnt[kPer];
-        int local = 0;
-#pragma unroll
-        for (int i = 0; i < kPer; ++i) {
-            const int b = lane * kPer + i;
-            int c = 0;
-            if (b < a.batch) {
-                // a context that does not fit the table is clipped to it instead of read out of bounds
-                const int ctx = min(max(a.context_lens[b], 0), a.max_blocks * kBlockSize);
-                sh_ctx[b] = ctx;
-                c = (ctx + kStageTok - 1) / kStageTok * hkv;
-            }
-            cnt[i] = c;
-            local += c;
-        }
-        int incl = local;                            // inclusive scan over the 64 lanes
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int up = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += up;
-        }
-        int run = incl - local;
-        if (lane == 0) sh_pref[0] = 0;
-#pragma unroll
-        for (int i = 0; i < kPer; ++i) {
-            run += cnt[i];
-            sh_pref[lane * kPer + i + 1] = run;      // entries past the batch repeat the total
-        }
-    }
-    __syncthreads();
-    const int64_t n_total = sh_pref[a.batch];
-    if (blockIdx.x == 0)
-        for (int i = threadIdx.x; i <= a.batch; i += kDecThreads) a.pref_out[i] = sh_pref[i];
-
-    // ---- sequences with no keys produce zero rows -----------------------------------------------
-    for (int b = blockIdx.x; b < a.batch; b += gridDim.x) {
-        if (sh_pref[b + 1] == sh_pref[b]) {
-            const int chunks = a.num_heads * kHeadDim / 8;
-            u32x4_t *dst = reinterpret_cast<u32x4_t *>(a.out + static_cast<int64_t>(b) * a.num_heads * kHeadDim);
-            for (int c = threadIdx.x; c < chunks; c += kDecThreads) dst[c] = u32x4_t{0u, 0u, 0u, 0u};
-        }
-    }
-
-    // With fewer stages than workers only the first n_total workers get (one) stage each, so that
-    // the workers of a pair are always consecutive.
     const int w = blockIdx.x * kDecWaves + wave;
-    const int64_t n_workers = n_total < kDecWorkers ? n_total : kDecWorkers;
-    if (w >= n_workers) return;                      // wave-uniform; no barrier follows
-    const int64_t lo = static_cast<int64_t>(w) * n_total / n_workers;
-    const int64_t hi = static_cast<int64_t>(w + 1) * n_total / n_workers;   // > lo
-
     u32x4_t *sK = lds + wave * kWaveLdsChunks;
     u32x4_t *sV = sK + kStageTok * 16;
     const int64_t row = static_cast<int64_t>(hkv) * kHeadDim;       // elements per token row
 
-    // ---- locate the first stage: largest b with sh_pref[b] <= lo --------------------------------
-    int b;
-    {
-        int l = 0, r = a.batch;                      // invariant: sh_pref[l] <= lo < sh_pref[r]
-        while (r - l > 1) {
-            const int mid = (l + r) >> 1;
-            if (sh_pref[mid] <= lo) l = mid; else r = mid;
-        }
-        b = l;
-    }
-    int nst = (sh_pref[b + 1] - sh_pref[b]) / hkv;   // stages per head of sequence b (> 0)
-    int g = static_cast<int>(lo - sh_pref[b]) / nst;
-    int s = static_cast<int>(lo - sh_pref[b]) % nst;
-
-    // HBM -> registers for stage (bb, gg, ss) of a sequence with nn stages per head.  Token rows
-    // are clamped to the last valid row of the stage, so only rows that were written are touched.
-    auto load_stage = [&](int bb, int gg, int ss, u32x4_t (&kr)[kStageLoads], u32x4_t (&vr)[kStageLoads],
-                          u32x4_t (&qr)[4], int &last) __attribute__((always_inline)) {
+    // Block and number of valid rows (minus one) of stage ss of sequence bb.
+    auto locate = [&](int bb, int ss, int32_t &blk, int &last) __attribute__((always_inline)) {
         last = min(kStageTok, sh_ctx[bb] - ss * kStageTok) - 1;                // in [0, 31]
-        int32_t blk = a.block_tables[static_cast<int64_t>(bb) * a.bt_row_stride + ss / kStagesPerBlock];
+        blk = a.block_tables[static_cast<int64_t>(bb) * a.bt_row_stride + ss / kStagesPerBlock];
         if (static_cast<uint32_t>(blk) >= static_cast<uint32_t>(a.num_blocks)) {
             blk = 0;                                  // bad table entry: contributes nothing
             last = -1;
         }
+    };
+    // HBM -> registers for stage ss of kv head gg of sequence bb, which lies in block blk.  Token
+    // rows are clamped to the last valid row of the stage, so only rows that were written are touched.
+    auto issue = [&](int bb, int gg, int ss, int32_t blk, int last, u32x4_t (&kr)[kStageLoads],
+                     u32x4_t (&vr)[kStageLoads], u32x4_t (&qr)[4]) __attribute__((always_inline)) {
         const int tok0 = (ss % kStagesPerBlock) * kStageTok;
         const int64_t base = (static_cast<int64_t>(blk) * kBlockSize + tok0) * row + gg * kHeadDim + r16 * 8;
         const bf16_t *kb = a.k_cache + base;
@@ -197,6 +140,125 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
             qr[i] = u;
         }
     };
+    auto load_stage = [&](int bb, int gg, int ss, u32x4_t (&kr)[kStageLoads], u32x4_t (&vr)[kStageLoads],
+                          u32x4_t (&qr)[4], int &last) __attribute__((always_inline)) {
+        int32_t blk;
+        locate(bb, ss, blk, last);
+        issue(bb, gg, ss, blk, last, kr, vr, qr);
+    };
+
+    u32x4_t kr[kStageLoads], vr[kStageLoads], qr[4];
+    int b, g, s, nst, last;
+    int64_t lo, hi;
+    if constexpr (kReuse) {
+        // ---- the split is in the workspace: first loads first, then the tables into LDS ---------
+        const int4 *rec = reinterpret_cast<const int4 *>(a.rec_out) + 2 * w;
+        const int4 r0 = rec[0], r1 = rec[1];
+        constexpr int kPer = kDecMaxBatch / kDecThreads;
+        int pv[kPer], cv[kPer];                          // table loads go out before the K/V loads
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int at = threadIdx.x + i * kDecThreads;
+            pv[i] = at < a.batch ? a.pref_out[at] : 0;
+            cv[i] = at < a.batch ? a.ctx_out[at] : 0;
+        }
+        const int total = a.pref_out[a.batch];
+        b = r0.x; g = r0.y; s = r0.z; nst = r0.w;
+        last = r1.y; lo = r1.z; hi = r1.w;
+        if (nst > 0) issue(b, g, s, r1.x, last, kr, vr, qr);
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int at = threadIdx.x + i * kDecThreads;
+            if (at < a.batch) {
+                sh_pref[at] = pv[i];
+                sh_ctx[at] = cv[i];
+            }
+        }
+        if (threadIdx.x == 0) sh_pref[a.batch] = total;
+        __syncthreads();
+    } else {
+        if (wave == 0) {
+            constexpr int kPer = kDecMaxBatch / kWave;  // 16 sequences per lane
+            int cnt[kPer];
+            int local = 0;
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                const int bi = lane * kPer + i;
+                int c = 0;
+                if (bi < a.batch) {
+                    // a context that does not fit the table is clipped to it instead of read out of bounds
+                    const int ctx = min(max(a.context_lens[bi], 0), a.max_blocks * kBlockSize);
+                    sh_ctx[bi] = ctx;
+                    c = (ctx + kStageTok - 1) / kStageTok * hkv;
+                }
+                cnt[i] = c;
+                local += c;
+            }
+            int incl = local;                            // inclusive scan over the 64 lanes
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int up = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += up;
+            }
+            int run = incl - local;
+            if (lane == 0) sh_pref[0] = 0;
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                run += cnt[i];
+                sh_pref[lane * kPer + i + 1] = run;      // entries past the batch repeat the total
+            }
+        }
+        __syncthreads();
+        if (blockIdx.x == 0) {
+            for (int i = threadIdx.x; i <= a.batch; i += kDecThreads) a.pref_out[i] = sh_pref[i];
+            for (int i = threadIdx.x; i < a.batch; i += kDecThreads) a.ctx_out[i] = sh_ctx[i];
+        }
+    }
+
+    // ---- sequences with no keys produce zero rows -----------------------------------------------
+    for (int bz = blockIdx.x; bz < a.batch; bz += gridDim.x) {
+        if (sh_pref[bz + 1] == sh_pref[bz]) {
+            const int chunks = a.num_heads * kHeadDim / 8;
+            u32x4_t *dst = reinterpret_cast<u32x4_t *>(a.out + static_cast<int64_t>(bz) * a.num_heads * kHeadDim);
+            for (int c = threadIdx.x; c < chunks; c += kDecThreads) dst[c] = u32x4_t{0u, 0u, 0u, 0u};
+        }
+    }
+
+    if constexpr (kReuse) {
+        if (nst == 0) return;                            // idle worker (wave-uniform; no barrier follows)
+    } else {
+        // With fewer stages than workers only the first n_total workers get (one) stage each, so that
+        // the workers of a pair are always consecutive.
+        const int64_t n_total = sh_pref[a.batch];
+        const int64_t n_workers = n_total < kDecWorkers ? n_total : kDecWorkers;
+        int4 *rec = reinterpret_cast<int4 *>(a.rec_out) + 2 * w;
+        if (w >= n_workers) {                            // wave-uniform; no barrier follows
+            if (lane == 0) rec[0] = int4{0, 0, 0, 0};
+            return;
+        }
+        lo = static_cast<int64_t>(w) * n_total / n_workers;
+        hi = static_cast<int64_t>(w + 1) * n_total / n_workers;   // > lo
+
+        // ---- locate the first stage: largest b with sh_pref[b] <= lo ----------------------------
+        {
+            int l = 0, r = a.batch;                      // invariant: sh_pref[l] <= lo < sh_pref[r]
+            while (r - l > 1) {
+                const int mid = (l + r) >> 1;
+                if (sh_pref[mid] <= lo) l = mid; else r = mid;
+            }
+            b = l;
+        }
+        nst = (sh_pref[b + 1] - sh_pref[b]) / hkv;       // stages per head of sequence b (> 0)
+        g = static_cast<int>(lo - sh_pref[b]) / nst;
+        s = static_cast<int>(lo - sh_pref[b]) % nst;
+        int32_t blk;
+        locate(b, s, blk, last);
+        issue(b, g, s, blk, last, kr, vr, qr);
+        if (lane == 0) {
+            rec[0] = int4{b, g, s, nst};
+            rec[1] = int4{blk, last, static_cast<int>(lo), static_cast<int>(hi)};
+        }
+    }
 
     f32x4_t oacc[8];               // O^T: lane = head r16, tile dt register i = dim 16dt + 4grp + i
     float m_run, l_run;
@@ -207,10 +269,6 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
         l_run = 0.f;
     };
     reset_state();
-
-    u32x4_t kr[kStageLoads], vr[kStageLoads], qr[4];
-    int last;
-    load_stage(b, g, s, kr, vr, qr, last);
 
     for (int64_t x = lo; x < hi; ++x) {
         // ---- registers -> LDS (swizzled) ------------------------------------------------------
@@ -389,8 +447,11 @@ __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArg
 }
 
 template <int G>
-static int launch_decode(const DecodeArgs &a, hipStream_t stream) {
-    hipLaunchKernelGGL(decode_stream_kernel<G>, dim3(kDecGrid), dim3(kDecThreads), 0, stream, a);
+static int launch_decode(const DecodeArgs &a, bool reuse, hipStream_t stream) {
+    if (reuse)
+        hipLaunchKernelGGL((decode_stream_kernel<G, true>), dim3(kDecGrid), dim3(kDecThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((decode_stream_kernel<G, false>), dim3(kDecGrid), dim3(kDecThreads), 0, stream, a);
     if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
     hipLaunchKernelGGL(decode_merge_kernel<G>, dim3(a.batch * a.num_kv_heads), dim3(G * kWave), 0, stream, a);
     return launch_status();
@@ -399,7 +460,7 @@ static int launch_decode(const DecodeArgs &a, hipStream_t stream) {
 static inline size_t align_up(size_t v, size_t to) { return (v + to - 1) / to * to; }
 
 struct DecodeWorkspace {
-    size_t pref_bytes, rows, total;
+    size_t pref_bytes, ctx_bytes, rec_bytes, rows, total;
 };
 static DecodeWorkspace decode_workspace(int32_t batch, int32_t num_heads, int32_t head_dim) {
     DecodeWorkspace ws;
@@ -408,7 +469,10 @@ static DecodeWorkspace decode_workspace(int32_t batch, int32_t num_heads, int32_
     // partial rows: one per query head of every (worker, pair) met along the stage list;
     // row index = (worker + pair) * G + head < W * G + batch * num_heads, and G <= 8
     ws.rows = static_cast<size_t>(kDecWorkers) * (num_heads < 8 ? num_heads : 8) + per_launch * num_heads;
-    ws.total = ws.pref_bytes + ws.rows * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
+    ws.ctx_bytes = align_up(per_launch * sizeof(int32_t), 256);
+    ws.rec_bytes = static_cast<size_t>(kDecWorkers) * 8 * sizeof(int32_t);
+    ws.total = ws.pref_bytes + ws.ctx_bytes + ws.rec_bytes +
+               ws.rows * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
     return ws;
 }
 
@@ -428,7 +492,21 @@ extern "C" int nva_paged_decode_attn(const void *q, int64_t q_row_stride, const 
                                      size_t workspace_bytes, int32_t batch, int32_t num_heads,
                                      int32_t num_kv_heads, int32_t head_dim, int32_t block_size,
                                      int32_t num_blocks, float scale, void *stream) {
+    return nva_paged_decode_attn_planned(q, q_row_stride, k_cache, v_cache, block_tables, bt_row_stride,
+                                         max_blocks, context_lens, out, workspace, workspace_bytes, batch,
+                                         num_heads, num_kv_heads, head_dim, block_size, num_blocks, scale,
+                                         NVA_PLAN_BUILD, stream);
+}
+
+extern "C" int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride, const void *k_cache,
+                                             const void *v_cache, const int32_t *block_tables,
+                                             int32_t bt_row_stride, int32_t max_blocks,
+                                             const int32_t *context_lens, void *out, void *workspace,
+                                             size_t workspace_bytes, int32_t batch, int32_t num_heads,
+                                             int32_t num_kv_heads, int32_t head_dim, int32_t block_size,
+                                             int32_t num_blocks, float scale, int32_t plan, void *stream) {
     using namespace nva;
+    if (plan != NVA_PLAN_BUILD && plan != NVA_PLAN_REUSE) return NVA_ERR_BAD_SHAPE;
     if (batch < 0 || num_heads <= 0 || num_kv_heads <= 0 || max_blocks < 0 || num_blocks < 0)
         return NVA_ERR_BAD_SHAPE;
     if (head_dim != kHeadDim || block_size != kBlockSize) return NVA_ERR_UNSUPPORTED_GEOMETRY;
@@ -455,7 +533,11 @@ extern "C" int nva_paged_decode_attn(const void *q, int64_t q_row_stride, const 
     a.bt_row_stride = bt_row_stride;
     a.q_row_stride = q_row_stride;
     a.pref_out = static_cast<int32_t *>(workspace);
-    a.part_ml = reinterpret_cast<float *>(static_cast<char *>(workspace) + ws.pref_bytes);
+    a.ctx_out = reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + ws.pref_bytes);
+    a.rec_out = reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + ws.pref_bytes + ws.ctx_bytes);
+    a.part_ml = reinterpret_cast<float *>(static_cast<char *>(workspace) + ws.pref_bytes + ws.ctx_bytes + ws.rec_bytes);
+    // every launch of a split batch overwrites the stored work split, so only a single launch can reuse it
+    const bool reuse = plan == NVA_PLAN_REUSE && batch <= kDecMaxBatch;
     a.part_o = a.part_ml + ws.rows * 2;
     a.max_blocks = max_blocks;
     a.num_heads = num_heads;
@@ -471,10 +553,10 @@ extern "C" int nva_paged_decode_attn(const void *q, int64_t q_row_stride, const 
         a.out = static_cast<bf16_t *>(out) + static_cast<int64_t>(b0) * num_heads * head_dim;
         int rc;
         switch (group) {
-            case 1: rc = launch_decode<1>(a, s); break;
-            case 2: rc = launch_decode<2>(a, s); break;
-            case 4: rc = launch_decode<4>(a, s); break;
-            default: rc = launch_decode<8>(a, s); break;
+            case 1: rc = launch_decode<1>(a, reuse, s); break;
+            case 2: rc = launch_decode<2>(a, reuse, s); break;
+            case 4: rc = launch_decode<4>(a, reuse, s); break;
+            default: rc = launch_decode<8>(a, reuse, s); break;
         }
         if (rc != NVA_OK) return rc;
     }

@@ -33,6 +33,8 @@ SIGNATURES = {
     "nva_paged_decode_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
     "nva_paged_decode_attn": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _sz,
                                         _i32, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
+    "nva_paged_decode_attn_planned": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _sz,
+                                                _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
     "nva_varlen_prefill_attn": (C.c_int, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32,
                                           _vp, _vp, _i32, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32,
                                           _f32, _vp]),

@@ -13,10 +13,11 @@ import torch
 from torch import nn
 
 from . import _lib
-from .context import get_context
+from .context import DecodePlan, get_context
 
 BLOCK_SIZE = 256
 _BF16 = torch.bfloat16
+_PLAN_BUILD, _PLAN_REUSE = 0, 1          # NVA_PLAN_BUILD / NVA_PLAN_REUSE of the C header
 
 
 def _stream() -> int:
@@ -81,12 +82,14 @@ def _decode_workspace(device, nbytes: int) -> torch.Tensor:
 
 def paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                            context_lens: torch.Tensor, block_tables: torch.Tensor, scale: float,
-                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           out: Optional[torch.Tensor] = None, plan: Optional[DecodePlan] = None) -> torch.Tensor:
     """One query token per sequence against its paged keys/values.
 
     ``q`` is ``[B, Hq, Dh]`` or ``[B, 1, Hq, Dh]``; the result has the shape of the
     reference's ``flash_attn_with_kvcache`` output, ``[B, 1, Hq, Dh]``
-    (nanovllm/layers/attention.py:72-74).
+    (nanovllm/layers/attention.py:72-74).  Calls that pass the same ``plan`` promise the same
+    ``context_lens``/``block_tables`` contents and run in order on one stream: the first
+    derives the work split, the others reuse it.
     """
     if q.dim() == 4:
         assert q.shape[1] == 1
@@ -111,11 +114,20 @@ def paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     lib = _lib.load()
     nbytes = lib.nva_paged_decode_workspace_bytes(b, hq, dh, max(max_blocks, 1))
     ws = _decode_workspace(q.device, nbytes)
-    rc = lib.nva_paged_decode_attn(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
-                                   block_tables.data_ptr(), block_tables.stride(0), max_blocks,
-                                   context_lens.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
-                                   b, hq, hkv, dh, block_size, num_blocks, float(scale), _stream())
-    _lib.check(rc, "nva_paged_decode_attn")
+    mode = _PLAN_BUILD
+    if plan is not None:
+        key = (ws.data_ptr(), b, hq, hkv, num_blocks, block_tables.data_ptr(), context_lens.data_ptr())
+        if plan.key is None:
+            plan.key = key
+        elif plan.key != key:
+            raise ValueError("decode plan reused with a different batch, geometry, table or workspace")
+        else:
+            mode = _PLAN_REUSE
+    rc = lib.nva_paged_decode_attn_planned(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+                                           block_tables.data_ptr(), block_tables.stride(0), max_blocks,
+                                           context_lens.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                           b, hq, hkv, dh, block_size, num_blocks, float(scale), mode, _stream())
+    _lib.check(rc, "nva_paged_decode_attn_planned")
     return out
 
 
@@ -192,4 +204,5 @@ class Attention(nn.Module):
                 q, k_cache if paged else k, v_cache if paged else v,
                 ctx.cu_seqlens_q, ctx.cu_seqlens_k, ctx.max_seqlen_q, ctx.max_seqlen_k,
                 self.scale, block_table=ctx.block_tables)
-        return paged_decode_attention(q, k_cache, v_cache, ctx.context_lens, ctx.block_tables, self.scale)
+        return paged_decode_attention(q, k_cache, v_cache, ctx.context_lens, ctx.block_tables, self.scale,
+                                      plan=getattr(ctx, "decode_plan", None))

@@ -14,6 +14,21 @@ from typing import Optional
 import torch
 
 
+class DecodePlan:
+    """Marks the decode-attention calls that share one work split: the layers of one decode
+    step, which see the same ``context_lens`` and ``block_tables``.  The first call made with
+    a plan derives the split, the later ones take it from the workspace.  A runner opts in by
+    putting a fresh plan on the context for every forward pass (and for every graph capture,
+    after the eager warm-up); without one every call derives its own split, which is what a
+    runner that reuses one ``Context`` for warm-up and capture (nanovllm/engine/model_runner.py:
+    229-237) needs.
+    """
+    __slots__ = ("key",)
+
+    def __init__(self):
+        self.key = None        # (workspace address, batch, heads, kv heads) of the call that built it
+
+
 @dataclass
 class Context:
     """Tensors describing the batch being run.  Index tensors are int32 on the device.
@@ -30,6 +45,7 @@ class Context:
     slot_mapping: Optional[torch.Tensor] = None
     context_lens: Optional[torch.Tensor] = None
     block_tables: Optional[torch.Tensor] = None
+    decode_plan: Optional[DecodePlan] = None     # not in the reference: see DecodePlan
 
 
 class _Holder:
@@ -41,9 +57,9 @@ def get_context() -> Context:
 
 
 def set_context(is_prefill, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=0, max_seqlen_k=0,
-                slot_mapping=None, context_lens=None, block_tables=None) -> None:
+                slot_mapping=None, context_lens=None, block_tables=None, decode_plan=None) -> None:
     _Holder.current = Context(is_prefill, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                              slot_mapping, context_lens, block_tables)
+                              slot_mapping, context_lens, block_tables, decode_plan)
 
 
 def reset_context() -> None:

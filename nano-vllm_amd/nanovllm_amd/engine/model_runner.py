@@ -15,7 +15,7 @@ import numpy as np
 import torch
 
 from .. import _lib
-from ..context import reset_context, set_context
+from ..context import DecodePlan, get_context, reset_context, set_context
 from ..sampler import Sampler
 from .config import EngineConfig
 from .model import Qwen3ForCausalLM
@@ -169,7 +169,7 @@ class ModelRunner:
         h = build_decode_inputs(seqs, self.block_size)
         set_context(False, slot_mapping=self._to_device(h["slot_mapping"], torch.int32),
                     context_lens=self._to_device(h["context_lens"], torch.int32),
-                    block_tables=self._to_device(h["block_tables"], torch.int32))
+                    block_tables=self._to_device(h["block_tables"], torch.int32), decode_plan=DecodePlan())
         return self._to_device(h["input_ids"], torch.int64), self._to_device(h["positions"], torch.int64)
 
     def prepare_sample(self, seqs: List[Sequence]) -> torch.Tensor:
@@ -298,6 +298,9 @@ class ModelRunner:
             set_context(False, slot_mapping=slot_mapping[:bs], context_lens=context_lens[:bs],
                         block_tables=block_tables[:bs])
             outputs[:bs] = self.model(input_ids[:bs], positions[:bs])        # eager warm-up (sizes workspaces)
+            # the captured layers share one work split of the decode kernel: the first layer derives
+            # it at every replay, the others take it from the workspace
+            get_context().decode_plan = DecodePlan()
             segments, hidden, residual = [], None, None
             for first, last in zip(cuts[:-1], cuts[1:]):
                 graph = torch.cuda.CUDAGraph()

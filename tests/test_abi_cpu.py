@@ -66,9 +66,10 @@ def test_store_kvcache_validation():
 def test_decode_validation_and_workspace_size():
     lib = _lib.load()
     ws = lib.nva_paged_decode_workspace_bytes
-    # prefix sums (256-byte aligned) + (2048 workers * min(heads, 8) + batch * heads) partial rows of 130 floats
-    assert ws(64, 16, 128, 8) == 512 + (2048 * 8 + 64 * 16) * 130 * 4
-    assert ws(3, 2, 128, 1) == 256 + (2048 * 2 + 3 * 2) * 130 * 4
+    # prefix sums and context lengths (each 256-byte aligned) + a 32-byte record per worker +
+    # (2048 workers * min(heads, 8) + batch * heads) partial rows of 130 floats
+    assert ws(64, 16, 128, 8) == 512 + 256 + 2048 * 32 + (2048 * 8 + 64 * 16) * 130 * 4
+    assert ws(3, 2, 128, 1) == 256 + 256 + 2048 * 32 + (2048 * 2 + 3 * 2) * 130 * 4
     assert ws(0, 16, 128, 8) == 0
     f = lib.nva_paged_decode_attn
     ok = dict(q=A, qs=2048, kc=A, vc=A, bt=A, bts=8, mb=8, cl=A, out=A, ws=A, wsb=ws(4, 16, 128, 8),
@@ -91,6 +92,13 @@ def test_decode_validation_and_workspace_size():
     assert call(wsb=ok["wsb"] - 1) == _lib.ERR_WORKSPACE_TOO_SMALL
     assert call(b=-2) == _lib.ERR_BAD_SHAPE
     assert call(b=0) == _lib.OK
+    g = lib.nva_paged_decode_attn_planned
+    a = ok
+    args = [a["q"], a["qs"], a["kc"], a["vc"], a["bt"], a["bts"], a["mb"], a["cl"], a["out"], a["ws"], a["wsb"],
+            a["b"], a["hq"], a["hkv"], a["dh"], a["bs"], a["nb"], a["scale"]]
+    assert g(*args, 2, None) == _lib.ERR_BAD_SHAPE                    # neither build nor reuse
+    assert g(*(args[:11] + [0] + args[12:]), 1, None) == _lib.OK      # empty batch
+    assert g(*(args[:9] + [A + 4] + args[10:]), 1, None) == _lib.ERR_MISALIGNED
 
 
 def test_prefill_validation():

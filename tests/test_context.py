@@ -9,8 +9,9 @@ import nanovllm_amd as nva
 
 def test_context_fields_and_defaults():
     names = [f.name for f in dataclasses.fields(nva.Context)]
+    # the reference's eight fields in its order (nanovllm/utils/context.py:7-15), then the one extension
     assert names == ["is_prefill", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k",
-                     "slot_mapping", "context_lens", "block_tables"]
+                     "slot_mapping", "context_lens", "block_tables", "decode_plan"]
     c = nva.Context()
     assert c.is_prefill is False and c.max_seqlen_q == 0 and c.max_seqlen_k == 0
     assert all(getattr(c, n) is None for n in names if n not in ("is_prefill", "max_seqlen_q", "max_seqlen_k"))

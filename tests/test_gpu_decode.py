@@ -5,6 +5,7 @@ import torch
 import oracle
 from nanovllm_amd import paged_decode_attention
 from nanovllm_amd import synthetic
+from nanovllm_amd.context import DecodePlan
 from helpers import assert_attn_close, bits
 
 pytestmark = pytest.mark.gpu
@@ -136,6 +137,52 @@ def test_decode_partials_are_fresh_across_calls(dev):
         i = it & 1
         out = paged_decode_attention(*dev_in[i], cases[i].scale)
         assert torch.equal(out, good[i]), f"iteration {it}"
+
+
+@pytest.mark.parametrize("shape", ["few_stages", "edge_lens", "many_splits", "config2"])
+def test_decode_plan_reuse_is_bit_identical(dev, shape):
+    """The layers of one decode step share context_lens and block_tables: the first call derives
+    the work split, the others reuse it from the workspace.  Both paths run the same arithmetic in
+    the same order, so the outputs are equal bit for bit, whatever q and caches a layer brings."""
+    if shape == "few_stages":         # fewer stages than workers: one stage per worker, idle workers
+        kw = dict(batch=5, num_blocks=64, ctx_lo=1, ctx_hi=300)
+    elif shape == "edge_lens":
+        kw = dict(num_blocks=64, context_lens=[0, 1, 2, 63, 64, 65, 255, 256, 257, 511, 512, 513, 1024, 0, 3])
+    elif shape == "many_splits":
+        kw = dict(batch=3, num_blocks=256, ctx_lo=9000, ctx_hi=12000)
+    else:
+        kw = {}
+    layers = [synthetic.decode_case(seed=60 + i, **kw) for i in range(3)]
+    ctx = layers[0].context_lens.to(dev)
+    tables = layers[0].block_tables.to(dev)
+    dev_in = [(c.q.to(dev), c.k_cache.to(dev), c.v_cache.to(dev)) for c in layers]
+    alone = [paged_decode_attention(*d, ctx, tables, layers[0].scale).clone() for d in dev_in]
+    want = oracle.paged_decode_attention(layers[0].q, layers[0].k_cache, layers[0].v_cache, layers[0].context_lens,
+                                         layers[0].block_tables, layers[0].scale, "fp32")
+    assert_attn_close(alone[0], want, shape)
+    for step in range(2):                                  # a second step rebuilds over the old records
+        plan = DecodePlan()
+        for d, good in zip(dev_in, alone):
+            out = paged_decode_attention(*d, ctx, tables, layers[0].scale, plan=plan)
+            assert torch.equal(out, good), (shape, step)
+    # a different batch after a plan was built: the next build must not see stale records
+    other = synthetic.decode_case(seed=70, batch=40, num_blocks=128, ctx_lo=1, ctx_hi=900)
+    od = (other.q.to(dev), other.k_cache.to(dev), other.v_cache.to(dev), other.context_lens.to(dev),
+          other.block_tables.to(dev))
+    o_alone = paged_decode_attention(*od, other.scale).clone()
+    plan = DecodePlan()
+    for _ in range(3):
+        assert torch.equal(paged_decode_attention(*od, other.scale, plan=plan), o_alone)
+
+
+def test_decode_plan_rejects_a_different_batch(dev):
+    case = synthetic.decode_case(seed=80, batch=6, num_blocks=64, ctx_lo=1, ctx_hi=600)
+    d = (case.q.to(dev), case.k_cache.to(dev), case.v_cache.to(dev), case.context_lens.to(dev),
+         case.block_tables.to(dev))
+    plan = DecodePlan()
+    paged_decode_attention(*d, case.scale, plan=plan)
+    with pytest.raises(ValueError):
+        paged_decode_attention(d[0][:4], d[1], d[2], d[3][:4], d[4][:4], case.scale, plan=plan)
 
 
 def test_decode_config5_full_size(dev):
