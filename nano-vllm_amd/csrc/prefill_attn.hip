@@ -34,6 +34,7 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));   // plain vectors
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x8_t __attribute__((ext_vector_type(8)));
 typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
+typedef __attribute__((address_space(3))) void *lds_void_ptr;
 
 constexpr int kPfThreads = 256;
 constexpr int kPfBM = 128;            // queries per workgroup
@@ -61,6 +62,16 @@ __device__ __forceinline__ float max3(float x, float y, float z) {
     float r;
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
     return r;
+}
+
+// global -> LDS without a register in between: lane l's 16 bytes at base + voff land at LDS byte
+// address lds_addr + 16 l.  Written as inline assembly on purpose: the compiler would make every
+// LDS read that follows its own builtin wait for the load (it cannot tell the two LDS buffers
+// apart), which would serialise the prefetch of the next tile with the arithmetic of this one.
+// The caller waits with s_waitcnt vmcnt(0) before the barrier that publishes the tile.
+__device__ __forceinline__ void load_to_lds_16(const void *base, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 
 template <bool kPaged>
@@ -128,16 +139,30 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         // (the column is clamped to the row: cu_seqlens_k is device data the host could not check)
         return kPaged ? a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + min((kt * kPfBN) >> 8, a.bt_row_stride - 1) + lane_zero] : 0;
     };
-    // Addressing: a tile's first row has a wave-uniform address; this lane's chunk of row
-    // tid/16 + 16*r sits a fixed 32-bit byte offset behind it, so a load needs no per-lane 64-bit
-    // arithmetic.  Only the last, partial tile clamps its rows to the last key.
-    const int lkey = tid >> 4, lch = tid & 15;
+    // K/V tiles go from global memory straight into LDS (global_load_lds_dwordx4: every lane
+    // moves 16 bytes, the 64 lanes of one instruction fill 1 KB of LDS in lane order -- four key
+    // rows -- and no vector register or LDS store instruction is spent on staging).  The LDS side
+    // of such a load cannot be permuted, so the XOR swizzle is applied on the global side: the lane
+    // that fills slot `lane % 16` of key row `key` fetches chunk slot ^ swizzle(key) of that row.
+    // Instruction r of wavefront w covers keys 16r + 4w + [0, 4): this lane's key is tid/16 + 16r.
+    // Addressing: a tile's first row has a wave-uniform address; this lane's chunk sits a fixed
+    // 32-bit byte offset behind it, so a load needs no per-lane 64-bit arithmetic.  Only the last,
+    // partial tile clamps its rows to the last key.
+    const int lkey = tid >> 4;
+    const int lch_k = (tid & 15) ^ (lkey & 15), lch_v = (tid & 15) ^ (4 * (lkey & 3));
     const int64_t kstride = kPaged ? static_cast<int64_t>(a.num_kv_heads) * kHeadDim : a.k_row_stride;
     const int64_t vstride = kPaged ? kstride : a.v_row_stride;
-    const uint32_t koff0 = static_cast<uint32_t>((lkey * kstride + lch * 8) * 2);
-    const uint32_t voff0 = static_cast<uint32_t>((lkey * vstride + lch * 8) * 2);
+    const uint32_t koff0 = static_cast<uint32_t>((lkey * kstride + lch_k * 8) * 2);
+    const uint32_t voff0 = static_cast<uint32_t>((lkey * vstride + lch_v * 8) * 2);
     const uint32_t kstep = static_cast<uint32_t>(16 * kstride * 2), vstep = static_cast<uint32_t>(16 * vstride * 2);
-    auto load_tile = [&](int kt, int32_t blk_v, u32x4_t (&kr)[4], u32x4_t (&vr)[4]) __attribute__((always_inline)) {
+    // LDS byte addresses of this wavefront's first 1 KB span in buffer 0 of each tensor
+    const uint32_t lds_k0 = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_ptr)&sK[0][wave * 64])));
+    const uint32_t lds_v0 = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_ptr)&sV[0][wave * 64])));
+    // Issues the loads of key tile kt into LDS buffer `buf`; returns false when the tile's block
+    // table entry is out of range (the loads then read block 0 and the tile is masked out).
+    auto load_tile = [&](int kt, int32_t blk_v, int buf) __attribute__((always_inline)) {
         const int32_t blk = kPaged ? __builtin_amdgcn_readfirstlane(blk_v) : 0;
         const bool ok = !kPaged || static_cast<uint32_t>(blk) < static_cast<uint32_t>(a.num_blocks);
         const int key0 = kt * kPfBN;
@@ -151,55 +176,44 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
             kb = reinterpret_cast<const char *>(a.k) + (static_cast<int64_t>(k0 + key0) * kstride + hkv * kHeadDim) * 2;
             vb = reinterpret_cast<const char *>(a.v) + (static_cast<int64_t>(k0 + key0) * vstride + hkv * kHeadDim) * 2;
         }
+        const uint32_t dk = lds_k0 + buf * (kPfTileChunks * 16), dv = lds_v0 + buf * (kPfTileChunks * 16);
         if (key0 + kPfBN <= lk) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                kr[r] = *reinterpret_cast<const u32x4_t *>(kb + r * kstep + koff0);
-                vr[r] = *reinterpret_cast<const u32x4_t *>(vb + r * vstep + voff0);
+                load_to_lds_16(kb, r * kstep + koff0, dk + r * 4096);
+                load_to_lds_16(vb, r * vstep + voff0, dv + r * 4096);
             }
         } else {
             const int last = lk - 1 - key0;              // >= 0: rows past it repeat it and are masked later
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = min(lkey + 16 * r, last);
-                kr[r] = *reinterpret_cast<const u32x4_t *>(kb + static_cast<uint32_t>((key * kstride + lch * 8) * 2));
-                vr[r] = *reinterpret_cast<const u32x4_t *>(vb + static_cast<uint32_t>((key * vstride + lch * 8) * 2));
+                load_to_lds_16(kb, static_cast<uint32_t>((key * kstride + lch_k * 8) * 2), dk + r * 4096);
+                load_to_lds_16(vb, static_cast<uint32_t>((key * vstride + lch_v * 8) * 2), dv + r * 4096);
             }
         }
         return ok;
     };
-    // registers -> LDS; a tile whose table entry was bad is stored as zeros (its keys then score
-    // 0 and its values add nothing)
-    auto store_tile = [&](int buf, bool ok, const u32x4_t (&kr)[4], const u32x4_t (&vr)[4]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int c = tid + kPfThreads * r;
-            const int key = c >> 4, ch = c & 15;
-            sK[buf][key * 16 + (ch ^ (key & 15))] = ok ? kr[r] : u32x4_t{0u, 0u, 0u, 0u};
-            sV[buf][key * 16 + (ch ^ (4 * (key & 3)))] = ok ? vr[r] : u32x4_t{0u, 0u, 0u, 0u};
-        }
-    };
 
-    u32x4_t kr[4], vr[4];
-    bool tile_ok = true;                                 // of the tile held in kr / vr
+    bool tile_ok = true;                                 // of the tile computed next
     int32_t blk_next = 0;                                // block id of the tile loaded next
-    if (ntiles > 0) tile_ok = load_tile(0, fetch_block(0), kr, vr);
+    if (ntiles > 0) tile_ok = load_tile(0, fetch_block(0), 0);
     if (ntiles > 1) blk_next = fetch_block(1);
     // Everything loaded so far (Q above all) is waited for here, and the Q fragments are then
     // passed through an empty asm.  Without this the compiler keeps treating them as in flight
     // inside the loop and makes each product wait for the loads issued just before it -- the
     // next tile's prefetch -- which put a full memory round trip into every tile.
-    __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
+    __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0): also the first tile has landed in LDS
 #pragma unroll
     for (int s = 0; s < 8; ++s) asm volatile("" : "+v"(qfrag[s]));
-    if (ntiles > 0) store_tile(0, tile_ok, kr, vr);
     __syncthreads();
 
     for (int kt = 0; kt < ntiles; ++kt) {
         const int buf = kt & 1;
         const bool more = kt + 1 < ntiles;
-        if (more) {                                      // in flight during this tile's arithmetic
-            tile_ok = load_tile(kt + 1, blk_next, kr, vr);
+        const bool cur_ok = tile_ok;
+        if (more) {                                      // lands in the other buffer during this tile's arithmetic
+            tile_ok = load_tile(kt + 1, blk_next, buf ^ 1);   // (that buffer was last read before the previous barrier)
             if (kt + 2 < ntiles) blk_next = fetch_block(kt + 2);
         }
 
@@ -221,8 +235,8 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         }
 
         // ---- causal mask, running softmax (base 2; the scale is folded into the exponent) -------
-        const int limit = qrow + off;                    // last key this query may see
-        if ((kt * kPfBN + kPfBN - 1) > (wave_qmin + off)) {   // only tiles that cross the diagonal
+        const int limit = cur_ok ? qrow + off : -1;      // last key this query may see
+        if ((kt * kPfBN + kPfBN - 1) > (wave_qmin + off) || !cur_ok) {   // only tiles that cross the diagonal
             const int key_base = kt * kPfBN + 4 * hh;
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2)
@@ -306,7 +320,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         }
 
         }
-        if (more) store_tile(buf ^ 1, tile_ok, kr, vr);           // the other buffer was last read before the previous barrier
+        __builtin_amdgcn_s_waitcnt(0x0F70);              // vmcnt(0): this wavefront's part of the next tile is in LDS
         __syncthreads();
     }
 
