@@ -74,6 +74,16 @@ __device__ __forceinline__ void load_to_lds_16(const void *base, uint32_t voff, 
                  :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 
+// The same, for operands that a matrix instruction has just written.  A vector instruction may
+// read the result registers of a v_mfma_f32_32x32x16_bf16 (8 passes) no sooner than 11 cycles
+// after its issue, and the hardware does not check: the compiler pads its own instructions with
+// s_nop, but it does not look inside inline assembly, so the padding is part of the statement.
+__device__ __forceinline__ float max3_after_mfma(float x, float y, float z) {
+    float r;
+    asm volatile("s_nop 7\n\ts_nop 2\n\tv_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
+    return r;
+}
+
 template <bool kPaged>
 __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const PrefillArgs a) {
     // Workgroups go to the 8 XCDs round-robin by linear id and every XCD has an L2 of its own, so
@@ -124,7 +134,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     const int q_hi = min(row0 + kPfBM, lq) - 1;          // last query row of the tile
     const int kv_end = min(lk, q_hi + off + 1);          // keys [0, kv_end) are visible to the tile
     const int ntiles = kv_end > 0 ? (kv_end + kPfBN - 1) / kPfBN : 0;
-    const int wave_qmin = row0 + wave * 32;
+    const int wave_qmin = row0 + __builtin_amdgcn_readfirstlane(wave) * 32;   // (in a scalar register: branches on it stay scalar)
 
     // global -> registers for key tile kt: thread t moves chunks t, t+256, t+512, t+768 of the tile
     // (chunk c = key c/16, 16 bytes c%16); keys past the end are clamped and masked later
@@ -244,15 +254,16 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
                 for (int i = 0; i < 16; ++i)
                     if (key_base + t2 * 32 + 8 * (i >> 2) + (i & 3) > limit) sacc[t2][i] = -INFINITY;
         }
-        float mloc0 = max3(sacc[0][0], sacc[0][1], sacc[0][2]), mloc1 = max3(sacc[1][0], sacc[1][1], sacc[1][2]);
-        mloc0 = max3(mloc0, sacc[0][3], sacc[0][4]);
-        mloc1 = max3(mloc1, sacc[1][3], sacc[1][4]);
+        // one dependent chain per sub-tile, so that every read of an accumulator follows the padded first one
+        float mloc0 = max3_after_mfma(sacc[0][0], sacc[0][1], sacc[0][2]);
+        float mloc1 = max3_after_mfma(sacc[1][0], sacc[1][1], sacc[1][2]);
 #pragma unroll
-        for (int i = 5; i < 15; i += 2) {
+        for (int i = 3; i < 15; i += 2) {
             mloc0 = max3(mloc0, sacc[0][i], sacc[0][i + 1]);
             mloc1 = max3(mloc1, sacc[1][i], sacc[1][i + 1]);
         }
-        const float mloc = max3(mloc0, mloc1, sacc[0][15] > sacc[1][15] ? sacc[0][15] : sacc[1][15]);
+        mloc1 = max3(mloc1, sacc[1][15], sacc[0][15]);   // (behind both padded reads)
+        const float mloc = max3(mloc0, mloc1, mloc1);
         // m_run is the reference point of the exponentials, p = exp2(scale*log2e * (s - m_run)).  It
         // follows the true running maximum lazily: only when the maximum has moved more than
         // kPfLazyLog2 powers of two past it are the sums rescaled (p stays below 2^kPfLazyLog2, far
