@@ -69,8 +69,11 @@ __device__ __forceinline__ float max3(float x, float y, float z) {
 // LDS read that follows its own builtin wait for the load (it cannot tell the two LDS buffers
 // apart), which would serialise the prefetch of the next tile with the arithmetic of this one.
 // The caller waits with s_waitcnt vmcnt(0) before the barrier that publishes the tile.
+// (s_nop 3: the load needs one wait state after the write of m0, and five after a vector
+// instruction wrote one of its scalar operands -- v_readfirstlane does -- which the compiler
+// cannot provide for an instruction it does not see.)
 __device__ __forceinline__ void load_to_lds_16(const void *base, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1"
                  :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 
