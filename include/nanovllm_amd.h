@@ -129,6 +129,8 @@ int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride,
  * block_tables != NULL: k/v are ignored (may be NULL) and every sequence reads its
  *   cu_seqlens_k[b+1]-cu_seqlens_k[b] logical positions from k_cache/v_cache through
  *   block_tables[b] (int32 [batch, max_blocks], row stride bt_row_stride, -1 padded).
+ *   A table entry outside [0, num_blocks) that a sequence's keys reach contributes nothing
+ *   (its 256 keys drop out) instead of faulting.
  * The causal mask is aligned to the END of the keys: query i of a sequence sees keys
  * j <= i + (Lk - Lq).  Empty query spans are no-ops.
  * out: bf16 [total_q, num_heads, head_dim] dense.  max_seqlen_q bounds the launch grid.

@@ -106,6 +106,30 @@ def test_prefill_empty_query_span_is_a_noop(dev):
     assert_attn_close(out, want, "empty span")
 
 
+def test_prefill_bad_table_entry_contributes_nothing(dev):
+    """A block-table entry outside [0, num_blocks) must neither fault nor add anything: the keys of
+    that block drop out.  Dropping whole prefix blocks leaves every remaining key visible to every
+    query, so the expected result is the oracle's for the same sequences with a shorter prefix."""
+    case = synthetic.prefill_case(seed=9, q_lens=[300, 150], prefix_blocks=[2, 1], num_blocks=32)
+    t = case.block_tables
+    bad = t.clone()
+    bad[0, 1] = 9999                                    # second prefix block of sequence 0
+    bad[1, 0] = -1                                      # the only prefix block of sequence 1
+    kc, vc = case.k_cache.to(dev), case.v_cache.to(dev)
+    store_kvcache(case.k.to(dev), case.v.to(dev), kc, vc, case.slot_mapping.to(dev))
+    out = varlen_prefill_attention(case.q.to(dev), kc, vc, case.cu_seqlens_q.to(dev), case.cu_seqlens_k.to(dev),
+                                   case.max_seqlen_q, case.max_seqlen_k, case.scale, block_table=bad.to(dev))
+    torch.cuda.synchronize()
+    ek, ev = case.k_cache.clone(), case.v_cache.clone()
+    oracle.store_kvcache(case.k, case.v, ek, ev, case.slot_mapping)
+    short = torch.full_like(t, -1)
+    short[0, :3] = torch.stack([t[0, 0], t[0, 2], t[0, 3]])     # 256 prefix keys, then the 300 new ones
+    short[1, :1] = t[1, 1]                                      # only the 150 new ones
+    cu_k = torch.tensor([0, 256 + 300, 256 + 300 + 150], dtype=torch.int32)
+    want = oracle.varlen_prefill_attention(case.q, None, None, case.cu_seqlens_q, cu_k, case.scale, ek, ev, short, "fp32")
+    assert_attn_close(out, want, "bad table entries")
+
+
 def test_prefill_sequences_do_not_leak(dev):
     case = synthetic.prefill_case(seed=6, batch=3, prefix_fraction=0.0, q_lo=50, q_hi=200)
     out, _ = _packed(case, dev)
