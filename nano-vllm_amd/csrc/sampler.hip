@@ -19,7 +19,8 @@
 // Pass 2 re-reads the logits (2 B/col) that pass 1 pulled through L2 / Infinity Cache.
 // With in-kernel noise there is nothing to replay against, so the draw uses the equivalent
 // Gumbel form argmax_i (x_i - log E_i), which needs no softmax: ONE pass over the logits
-// (sampler_gumbel_kernel) followed by the per-row pick -- the same exact categorical draw.
+// (sampler_gumbel_kernel, chunks of 8192 columns) followed by the per-row pick -- the same exact
+// categorical draw.
 // Algorithmic HBM bytes per row: vocab * 2 B (+ vocab * 4 B when the noise is read).
 #include "nva_common.h"
 
@@ -196,6 +197,15 @@ __global__ __launch_bounds__(kSampThreads) void sampler_argmax_kernel(
 // In-kernel noise: score_i = logit_i * log2(e)/T - log2(-log2(u_i)), u_i uniform in (0,1) from Philox.
 // (E_i = -ln(u_i); log2(E_i) = log2(-log2(u_i)) + const, and constants do not move the argmax.)
 // Greedy rows (T == 0) use score_i = logit_i.
+// One pass over the logits with in-kernel noise.  A workgroup takes kGumbelChunk columns of one
+// row: every lane issues its kGumbelVec 16-byte loads up front, then scores 8 columns per load.
+// (Four loads per lane instead of one: the cross-lane reduction and the per-workgroup overhead are
+// paid once per 8192 columns instead of once per 2048 -- they were a quarter of the kernel.)
+constexpr int kGumbelVec = 4;
+constexpr int kGumbelChunk = kSampChunk * kGumbelVec;
+
+__host__ __device__ inline int gumbel_chunks(int vocab) { return (vocab + kGumbelChunk - 1) / kGumbelChunk; }
+
 __global__ __launch_bounds__(kSampThreads) void sampler_gumbel_kernel(
     const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
     uint64_t seed, uint64_t offset, float *__restrict__ part_best, int32_t *__restrict__ part_idx,
@@ -208,36 +218,50 @@ __global__ __launch_bounds__(kSampThreads) void sampler_gumbel_kernel(
     const float t_in = temperatures[b];
     const bool greedy = (t_in == 0.f);
     const float k = greedy ? 1.f : 1.4426950408889634f / t_in;
-    const int col0 = chunk * kSampChunk + threadIdx.x * 8;
-    float x[8];
-    if (vec_ok && col0 + 8 <= vocab) {
-        unpack8(*reinterpret_cast<const uint4 *>(row + col0), x);
-    } else {
+    uint4 raw[kGumbelVec];
+    int col0[kGumbelVec];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = (col0 + i < vocab) ? bf16_to_f32(row[col0 + i]) : -INFINITY;
+    for (int v = 0; v < kGumbelVec; ++v) {
+        col0[v] = chunk * kGumbelChunk + v * kSampChunk + threadIdx.x * 8;
+        raw[v] = make_uint4(0u, 0u, 0u, 0u);
+        if (vec_ok && col0[v] + 8 <= vocab) raw[v] = *reinterpret_cast<const uint4 *>(row + col0[v]);
     }
-    float g[8];
-    if (greedy) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) g[i] = 0.f;
-    } else {
-        const uint2 key = make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
-        const uint32_t o_lo = static_cast<uint32_t>(offset), o_hi = static_cast<uint32_t>(offset >> 32);
-        const uint4 r0 = Philox::draw(make_uint4(static_cast<uint32_t>(col0 >> 2), b, o_lo, o_hi), key);
-        const uint4 r1 = Philox::draw(make_uint4(static_cast<uint32_t>(col0 >> 2) + 1u, b, o_lo, o_hi), key);
-        const uint32_t r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            // u in (0, 1): 23 random bits plus one half, so that neither log below sees 0 or 1
-            const float u = (static_cast<float>(r[i] >> 9) + 0.5f) * 1.1920928955078125e-7f;
-            g[i] = __builtin_amdgcn_logf(-__builtin_amdgcn_logf(u));      // log2(-log2 u)
-        }
-    }
+    const uint2 key = make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+    const uint32_t o_lo = static_cast<uint32_t>(offset), o_hi = static_cast<uint32_t>(offset >> 32);
     float best = -INFINITY;
     int best_i = 0x7fffffff;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-        if (col0 + i < vocab) better(best, best_i, fmaf(x[i], k, -g[i]), col0 + i);
+    for (int v = 0; v < kGumbelVec; ++v) {
+        if (col0[v] >= vocab) continue;
+        float x[8];
+        if (vec_ok && col0[v] + 8 <= vocab) {
+            unpack8(raw[v], x);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = (col0[v] + i < vocab) ? bf16_to_f32(row[col0[v] + i]) : -INFINITY;
+        }
+        float g[8];
+        if (greedy) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) g[i] = 0.f;
+        } else {
+            const uint4 r0 = Philox::draw(make_uint4(static_cast<uint32_t>(col0[v] >> 2), b, o_lo, o_hi), key);
+            const uint4 r1 = Philox::draw(make_uint4(static_cast<uint32_t>(col0[v] >> 2) + 1u, b, o_lo, o_hi), key);
+            const uint32_t r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                // u in (0, 1): 23 random bits plus one half, so that neither log below sees 0 or 1
+                const float u = (static_cast<float>(r[i] >> 9) + 0.5f) * 1.1920928955078125e-7f;
+                g[i] = __builtin_amdgcn_logf(-__builtin_amdgcn_logf(u));      // log2(-log2 u)
+            }
+        }
+        // columns are visited in increasing order, so a strict comparison keeps the lowest column on ties
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float sc = fmaf(x[i], k, -g[i]);
+            if (col0[v] + i < vocab && sc > best) { best = sc; best_i = col0[v] + i; }
+        }
+    }
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
         const float os = __shfl_xor(best, off, 64);
@@ -302,11 +326,12 @@ extern "C" int nva_sample(const void *logits, int64_t logits_row_stride, const f
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bf16_t *lg = static_cast<const bf16_t *>(logits);
     if (noise == nullptr) {
-        hipLaunchKernelGGL(sampler_gumbel_kernel, dim3(nchunks, batch), dim3(kSampThreads), 0, s, lg,
-                           logits_row_stride, temperatures, seed, offset, part_best, part_idx, vocab, nchunks);
+        const int gchunks = gumbel_chunks(vocab);              // fewer, wider chunks: fits the same workspace
+        hipLaunchKernelGGL(sampler_gumbel_kernel, dim3(gchunks, batch), dim3(kSampThreads), 0, s, lg,
+                           logits_row_stride, temperatures, seed, offset, part_best, part_idx, vocab, gchunks);
         if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
         hipLaunchKernelGGL(sampler_pick_kernel, dim3(batch), dim3(kWave), 0, s, part_best, part_idx, out_tokens,
-                           nchunks);
+                           gchunks);
         return launch_status();
     }
     hipLaunchKernelGGL(sampler_partials_kernel, dim3(nchunks, batch), dim3(kSampThreads), 0, s, lg,
