@@ -175,6 +175,19 @@ def test_decode_plan_reuse_is_bit_identical(dev, shape):
         assert torch.equal(paged_decode_attention(*od, other.scale, plan=plan), o_alone)
 
 
+def test_decode_batch_above_one_launch(dev):
+    """More than 1024 sequences run as two launches sharing the workspace; a stored work split is
+    then never reused (each launch overwrites it), with or without a plan object."""
+    case = synthetic.decode_case(seed=81, batch=1100, num_heads=2, num_kv_heads=1, num_blocks=1200, ctx_lo=1, ctx_hi=256)
+    d = (case.q.to(dev), case.k_cache.to(dev), case.v_cache.to(dev), case.context_lens.to(dev),
+         case.block_tables.to(dev))
+    out = paged_decode_attention(*d, case.scale).clone()
+    assert_attn_close(out, _oracle(case), "batch 1100")
+    plan = DecodePlan()
+    for _ in range(3):
+        assert torch.equal(paged_decode_attention(*d, case.scale, plan=plan), out)
+
+
 def test_decode_plan_rejects_a_different_batch(dev):
     case = synthetic.decode_case(seed=80, batch=6, num_blocks=64, ctx_lo=1, ctx_hi=600)
     d = (case.q.to(dev), case.k_cache.to(dev), case.v_cache.to(dev), case.context_lens.to(dev),
