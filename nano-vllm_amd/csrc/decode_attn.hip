@@ -432,6 +432,9 @@ __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArg
     mx = wave_max(mx);
     float acc0 = 0.f, acc1 = 0.f, lsum = 0.f;
     if (mx > -INFINITY) {
+        // eight partials in flight per lane: a pair met by many workers (small batches) is otherwise one dependent
+        // memory round trip per partial (measured: 22 -> 18 us per call at batch 16; more unrolling is slower again)
+#pragma unroll 8
         for (int pi = 0; pi < n_parts; ++pi) {
             const int64_t at = row0 + static_cast<int64_t>(pi) * G;
             const float f = exp2f(a.part_ml[at * 2] - mx);
