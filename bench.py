@@ -196,13 +196,13 @@ def bench_sampler(args, dev):
     alg = batch * vocab * 2
     gbps = alg / (per_step_ms * 1e-3) / 1e9
     result = {
-        "metric": "sampler (in-kernel noise), achieved HBM GB/s", "value": round(gbps, 1), "unit": "GB/s",
+        "metric": "sampler (in-kernel randomness), achieved HBM GB/s", "value": round(gbps, 1), "unit": "GB/s",
         "ms_per_step": round(per_step_ms, 5),
-        "config": {"workload": "sampler: 256 rows x 151,936 bf16 logits, T=0.6, Philox noise in-kernel",
+        "config": {"workload": "sampler: 256 rows x 151,936 bf16 logits, T=0.6, in-kernel randomness (one uniform per row, inverse CDF)",
                    "batch": batch},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "sampler_gumbel_kernel + sampler_pick_kernel",
+                     "kernel": "sampler_cdf_sums_kernel + sampler_cdf_select_kernel",
                      "algorithmic_bytes_per_launch": alg},
     }
 

@@ -156,8 +156,11 @@ int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride,
  * logits: bf16 [batch, vocab], row stride logits_row_stride elements.
  * temperatures: fp32 [batch].  T == 0 selects greedy argmax(logits) for that row (an
  * extension; the reference forbids T <= 1e-10, nanovllm/sampling_params.py:11).
- * noise: fp32 [batch, vocab] Exp(1) draws (row stride noise_row_stride), or NULL to draw
- * them inside the kernel from Philox4x32-10 keyed by (seed, offset, row, column).
+ * noise: fp32 [batch, vocab] Exp(1) draws (row stride noise_row_stride): the formula above is
+ * evaluated as written and a draw can be replayed.  NULL: the token is drawn from the same
+ * categorical distribution softmax(logits / T) by inverse CDF (first column whose running sum of
+ * probabilities exceeds u), with one uniform u per row from Philox4x32-10 keyed by
+ * (seed, offset, row); the same (seed, offset) reproduces the draw.
  * out_tokens: int64 [batch].
  * workspace: at least nva_sample_workspace_bytes() bytes, 16-byte aligned.
  */

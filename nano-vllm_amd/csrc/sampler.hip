@@ -1,26 +1,24 @@
-// Temperature / exponential-race sampler for gfx950.
+// Temperature sampler for gfx950.
 //
 // Replaces Sampler.forward of nanovllm/layers/sampler.py:10-15:
 //     x = float(logits) / T;  p = softmax(x);  token = argmax_i p_i / max(E_i, 1e-10)
-// E ~ Exp(1) is either read from a caller-supplied tensor (replayable; used for parity) or
-// drawn in-kernel from Philox4x32-10 (no noise traffic).  The arithmetic keeps the
-// reference's operation order -- true fp32 division by T, exp(x - rowmax) / rowsum, then the
-// division by the clamped noise -- so the argmax can only differ from the reference where
-// two scores are equal to within fp32 rounding.
+// With a caller-supplied tensor of E ~ Exp(1) draws (replayable; used for parity) the arithmetic
+// keeps the reference's operation order -- true fp32 division by T, exp(x - rowmax) / rowsum, then
+// the division by the clamped noise -- so the argmax can only differ from the reference where two
+// scores are equal to within fp32 rounding.  Without one (what serving uses) the token is drawn
+// from the same categorical distribution by inverse CDF with one in-kernel uniform per row.
 //
 // A row of 151,936 logits is far too little work for one workgroup and 64..256 rows are
-// too few workgroups for 256 CUs, so a row is cut into chunks of 2048 columns (one
-// workgroup of 256 lanes, one 16-byte load of 8 bf16 per lane):
-// With a caller-supplied noise tensor (the replayable form):
+// too few workgroups for 256 CUs, so a row is cut into chunks (one workgroup of 256 lanes each,
+// 16-byte loads of 8 bf16 per lane).
+// With a caller-supplied noise tensor, chunks of 2048 columns:
 //   pass 1  per (chunk, row): chunk max and sum exp(x - chunk max)          -> workspace
 //   pass 2  per (chunk, row): merge the row's partials into (max, sum), then
 //           best p_i / E_i and its column inside the chunk                   -> workspace
 //   pass 3  per row: best chunk, lowest column on ties                       -> int64 token
 // Pass 2 re-reads the logits (2 B/col) that pass 1 pulled through L2 / Infinity Cache.
-// With in-kernel noise there is nothing to replay against, so the draw uses the equivalent
-// Gumbel form argmax_i (x_i - log E_i), which needs no softmax: ONE pass over the logits
-// (sampler_gumbel_kernel, chunks of 8192 columns) followed by the per-row pick -- the same exact
-// categorical draw.
+// Without noise, chunks of 8192 columns: one pass for the chunk sums, then a per-row selection
+// that re-reads a single chunk (see sampler_cdf_sums_kernel below).
 // Algorithmic HBM bytes per row: vocab * 2 B (+ vocab * 4 B when the noise is read).
 #include "nva_common.h"
 
@@ -194,22 +192,46 @@ __global__ __launch_bounds__(kSampThreads) void sampler_argmax_kernel(
     }
 }
 
-// In-kernel noise: score_i = logit_i * log2(e)/T - log2(-log2(u_i)), u_i uniform in (0,1) from Philox.
-// (E_i = -ln(u_i); log2(E_i) = log2(-log2(u_i)) + const, and constants do not move the argmax.)
-// Greedy rows (T == 0) use score_i = logit_i.
-// One pass over the logits with in-kernel noise.  A workgroup takes kGumbelChunk columns of one
-// row: every lane issues its kGumbelVec 16-byte loads up front, then scores 8 columns per load.
-// (Four loads per lane instead of one: the cross-lane reduction and the per-workgroup overhead are
-// paid once per 8192 columns instead of once per 2048 -- they were a quarter of the kernel.)
-constexpr int kGumbelVec = 4;
-constexpr int kGumbelChunk = kSampChunk * kGumbelVec;
+// ---- in-kernel randomness: one uniform per row, inverse-CDF draw -----------------------------
+// Without a noise tensor to replay against, the exponential race is replaced by the textbook
+// draw from the same categorical distribution: with w_i = exp2((x_i - M) * log2(e)/T) and one
+// uniform u per row, the token is the first i (in column order) whose running sum of w exceeds
+// u * sum(w).  One Philox call per ROW instead of one random number and two logarithms per
+// column leaves a multiply, an exponential and an add per column -- the pass over the logits
+// runs at memory speed.
+//   pass A  per (8192-column chunk, row): chunk max m_c, s_c = sum exp2(y - m_c), and the chunk's
+//           arg-max (used by temperature-0 rows)                                -> workspace
+//   pass B  per row: M = max m_c, chunk weights s_c * exp2(m_c - M), their running sum picks
+//           the chunk; its 8192 logits are read once more (32 consecutive columns per lane), a
+//           workgroup scan picks the lane and the lane walks its columns        -> int64 token
+// Rounding can leave the target a hair beyond the last running sum; it then falls on the last
+// column of positive weight.  A row without any finite logit yields token 0.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kCdfVec = 4;                                    // 16-byte loads per lane in pass A
+constexpr int kCdfChunk = kSampChunk * kCdfVec;               // 8192 columns per workgroup
 
-__host__ __device__ inline int gumbel_chunks(int vocab) { return (vocab + kGumbelChunk - 1) / kGumbelChunk; }
+__host__ __device__ inline int cdf_chunks(int vocab) { return (vocab + kCdfChunk - 1) / kCdfChunk; }
 
-__global__ __launch_bounds__(kSampThreads) void sampler_gumbel_kernel(
+__device__ __forceinline__ float block_max4(float v, float *sh, int lane, int wave) {
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) sh[wave] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+}
+
+__device__ __forceinline__ float block_sum4(float v, float *sh, int lane, int wave) {
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) sh[wave] = v;
+    __syncthreads();
+    return (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
+
+__global__ __launch_bounds__(kSampThreads) void sampler_cdf_sums_kernel(
     const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
-    uint64_t seed, uint64_t offset, float *__restrict__ part_best, int32_t *__restrict__ part_idx,
-    int32_t vocab, int32_t nchunks) {
+    float *__restrict__ part_max, float *__restrict__ part_sum, float *__restrict__ part_best,
+    int32_t *__restrict__ part_idx, int32_t vocab, int32_t nchunks) {
     const int chunk = blockIdx.x;
     const int b = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -218,64 +240,210 @@ __global__ __launch_bounds__(kSampThreads) void sampler_gumbel_kernel(
     const float t_in = temperatures[b];
     const bool greedy = (t_in == 0.f);
     const float k = greedy ? 1.f : 1.4426950408889634f / t_in;
-    uint4 raw[kGumbelVec];
-    int col0[kGumbelVec];
+    u32x4_t raw[kCdfVec];
+    int col0[kCdfVec];
 #pragma unroll
-    for (int v = 0; v < kGumbelVec; ++v) {
-        col0[v] = chunk * kGumbelChunk + v * kSampChunk + threadIdx.x * 8;
-        raw[v] = make_uint4(0u, 0u, 0u, 0u);
-        if (vec_ok && col0[v] + 8 <= vocab) raw[v] = *reinterpret_cast<const uint4 *>(row + col0[v]);
+    for (int v = 0; v < kCdfVec; ++v) {
+        col0[v] = chunk * kCdfChunk + v * kSampChunk + threadIdx.x * 8;
+        raw[v] = u32x4_t{0u, 0u, 0u, 0u};
+        // (streamed once: non-temporal, so that the rows do not displace one another in L2)
+        if (vec_ok && col0[v] + 8 <= vocab) raw[v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row + col0[v]));
     }
-    const uint2 key = make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
-    const uint32_t o_lo = static_cast<uint32_t>(offset), o_hi = static_cast<uint32_t>(offset >> 32);
-    float best = -INFINITY;
-    int best_i = 0x7fffffff;
+    float y[kCdfVec][8];
+    float m = -INFINITY;
 #pragma unroll
-    for (int v = 0; v < kGumbelVec; ++v) {
-        if (col0[v] >= vocab) continue;
-        float x[8];
+    for (int v = 0; v < kCdfVec; ++v) {
         if (vec_ok && col0[v] + 8 <= vocab) {
-            unpack8(raw[v], x);
+            unpack8(make_uint4(raw[v][0], raw[v][1], raw[v][2], raw[v][3]), y[v]);
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[i] = (col0[v] + i < vocab) ? bf16_to_f32(row[col0[v] + i]) : -INFINITY;
+            for (int i = 0; i < 8; ++i) y[v][i] = (col0[v] + i < vocab) ? bf16_to_f32(row[col0[v] + i]) : -INFINITY;
         }
-        float g[8];
-        if (greedy) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) g[i] = 0.f;
-        } else {
-            const uint4 r0 = Philox::draw(make_uint4(static_cast<uint32_t>(col0[v] >> 2), b, o_lo, o_hi), key);
-            const uint4 r1 = Philox::draw(make_uint4(static_cast<uint32_t>(col0[v] >> 2) + 1u, b, o_lo, o_hi), key);
-            const uint32_t r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                // u in (0, 1): 23 random bits plus one half, so that neither log below sees 0 or 1
-                const float u = (static_cast<float>(r[i] >> 9) + 0.5f) * 1.1920928955078125e-7f;
-                g[i] = __builtin_amdgcn_logf(-__builtin_amdgcn_logf(u));      // log2(-log2 u)
-            }
-        }
-        // columns are visited in increasing order, so a strict comparison keeps the lowest column on ties
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float sc = fmaf(x[i], k, -g[i]);
-            if (col0[v] + i < vocab && sc > best) { best = sc; best_i = col0[v] + i; }
+            y[v][i] *= k;
+            m = fmaxf(m, y[v][i]);
         }
-    }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float os = __shfl_xor(best, off, 64);
-        const int oi = __shfl_xor(best_i, off, 64);
-        better(best, best_i, os, oi);
     }
     __shared__ float sh[4];
     __shared__ int shi[4];
-    if (lane == 0) { sh[wave] = best; shi[wave] = best_i; }
+    if (greedy) {                                        // row-uniform branch: chunk arg-max, lowest column on ties
+        float best = -INFINITY;
+        int best_i = 0x7fffffff;
+#pragma unroll
+        for (int v = 0; v < kCdfVec; ++v)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (col0[v] + i < vocab && y[v][i] > best) { best = y[v][i]; best_i = col0[v] + i; }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const float os = __shfl_xor(best, off, 64);
+            const int oi = __shfl_xor(best_i, off, 64);
+            better(best, best_i, os, oi);
+        }
+        if (lane == 0) { sh[wave] = best; shi[wave] = best_i; }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (int w = 1; w < 4; ++w) better(best, best_i, sh[w], shi[w]);
+            part_best[static_cast<int64_t>(b) * nchunks + chunk] = best;
+            part_idx[static_cast<int64_t>(b) * nchunks + chunk] = best_i;
+        }
+        return;
+    }
+    m = block_max4(m, sh, lane, wave);
+    const float mm = (m == -INFINITY) ? 0.f : m;           // a chunk of -inf logits sums to 0
+    float ssum = 0.f;
+#pragma unroll
+    for (int v = 0; v < kCdfVec; ++v) {
+        float part = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) part += __builtin_amdgcn_exp2f(y[v][i] - mm);     // exp2(-inf) = 0 past the row end
+        ssum += part;
+    }
+    ssum = block_sum4(ssum, sh, lane, wave);
+    if (threadIdx.x == 0) {
+        part_max[static_cast<int64_t>(b) * nchunks + chunk] = m;
+        part_sum[static_cast<int64_t>(b) * nchunks + chunk] = ssum;
+    }
+}
+
+__global__ __launch_bounds__(kSampThreads) void sampler_cdf_select_kernel(
+    const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
+    uint64_t seed, uint64_t offset, const float *__restrict__ part_max, const float *__restrict__ part_sum,
+    const float *__restrict__ part_best, const int32_t *__restrict__ part_idx,
+    int64_t *__restrict__ out_tokens, int32_t vocab, int32_t nchunks) {
+    const int b = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float t_in = temperatures[b];
+    __shared__ float sh[4];
+    __shared__ int sh_pick[1];
+    if (t_in == 0.f) {                                   // greedy: best chunk, lowest column on ties
+        if (wave == 0) {
+            float best = -INFINITY;
+            int best_i = 0x7fffffff;
+            for (int c = lane; c < nchunks; c += kWave)
+                better(best, best_i, part_best[static_cast<int64_t>(b) * nchunks + c],
+                       part_idx[static_cast<int64_t>(b) * nchunks + c]);
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const float os = __shfl_xor(best, off, 64);
+                const int oi = __shfl_xor(best_i, off, 64);
+                better(best, best_i, os, oi);
+            }
+            if (lane == 0) out_tokens[b] = (best_i == 0x7fffffff) ? 0 : static_cast<int64_t>(best_i);
+        }
+        return;
+    }
+    const float k = 1.4426950408889634f / t_in;
+    // ---- row maximum and the chunk weights relative to it -------------------------------------
+    float m = -INFINITY;
+    for (int c = threadIdx.x; c < nchunks; c += kSampThreads)
+        m = fmaxf(m, part_max[static_cast<int64_t>(b) * nchunks + c]);
+    m = block_max4(m, sh, lane, wave);
+    if (m == -INFINITY) {                                // no finite logit in the row
+        if (threadIdx.x == 0) out_tokens[b] = 0;
+        return;
+    }
+    // one uniform per row, in (0, 1): 24 random bits plus one half
+    const uint2 key = make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+    const uint4 r = Philox::draw(make_uint4(static_cast<uint32_t>(b), 0x5a17u, static_cast<uint32_t>(offset),
+                                            static_cast<uint32_t>(offset >> 32)), key);
+    const float u = (static_cast<float>(r.x >> 8) + 0.5f) * 5.9604644775390625e-8f;
+    // chunk weights into LDS (all lanes), then one lane walks them: running sum in chunk order
+    constexpr int kLdsChunks = 1024;                     // rows with more chunks walk the workspace instead
+    __shared__ float sh_w[kLdsChunks];
+    const bool in_lds = nchunks <= kLdsChunks;
+    if (in_lds)
+        for (int c = threadIdx.x; c < nchunks; c += kSampThreads) {
+            const int64_t at = static_cast<int64_t>(b) * nchunks + c;
+            sh_w[c] = part_sum[at] * __builtin_amdgcn_exp2f(part_max[at] - m);
+        }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; ++w) better(best, best_i, sh[w], shi[w]);
-        part_best[static_cast<int64_t>(b) * nchunks + chunk] = best;
-        part_idx[static_cast<int64_t>(b) * nchunks + chunk] = best_i;
+        auto weight = [&](int c) {
+            const int64_t at = static_cast<int64_t>(b) * nchunks + c;
+            return in_lds ? sh_w[c] : part_sum[at] * __builtin_amdgcn_exp2f(part_max[at] - m);
+        };
+        float total = 0.f;
+        for (int c = 0; c < nchunks; ++c) total += weight(c);
+        const float target = u * total;
+        float run = 0.f, before = 0.f;
+        int pick = -1, last_live = 0;
+        for (int c = 0; c < nchunks; ++c) {
+            const float w = weight(c);
+            if (w > 0.f) last_live = c;
+            if (pick < 0 && w > 0.f && run + w > target) { pick = c; before = run; }
+            run += w;
+        }
+        float rest_in_chunk = target - before;                   // what is left to walk inside the chunk
+        if (pick < 0) { pick = last_live; rest_in_chunk = INFINITY; }   // rounding: beyond the last running sum
+        sh_pick[0] = pick;
+        sh[0] = rest_in_chunk;
+    }
+    __syncthreads();
+    const int chunk = sh_pick[0];
+    const float rest = sh[0];
+    __syncthreads();
+    // ---- inside the chunk: 32 consecutive columns per lane, scan over the 256 lanes -------------
+    const bf16_t *row = logits + static_cast<int64_t>(b) * row_stride;
+    const int c0 = chunk * kCdfChunk + threadIdx.x * 32;
+    float w[32];
+    float mine = 0.f;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        float x[8];
+        const int cc = c0 + v * 8;
+        if (((reinterpret_cast<uintptr_t>(row + cc) & 15u) == 0) && cc + 8 <= vocab) {
+            unpack8(*reinterpret_cast<const uint4 *>(row + cc), x);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = (cc + i < vocab) ? bf16_to_f32(row[cc + i]) : -INFINITY;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            w[v * 8 + i] = __builtin_amdgcn_exp2f(x[i] * k - m);
+            mine += w[v * 8 + i];
+        }
+    }
+    // inclusive scan of `mine` over the workgroup, in lane order
+    float incl = mine;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float up = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += up;
+    }
+    if (lane == 63) sh[wave] = incl;
+    __syncthreads();
+    for (int wv = 0; wv < wave; ++wv) incl += sh[wv];
+    // owner: the first lane whose running sum exceeds `rest` (its span then contains it); if rounding
+    // put `rest` beyond the chunk's total, the last lane of positive weight
+    int first = (mine > 0.f && incl > rest) ? static_cast<int>(threadIdx.x) : 0x7fffffff;
+    int live = (mine > 0.f) ? static_cast<int>(threadIdx.x) : -1;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        first = min(first, __shfl_xor(first, off, 64));
+        live = max(live, __shfl_xor(live, off, 64));
+    }
+    __shared__ int sh_first[4], sh_live[4];
+    if (lane == 0) { sh_first[wave] = first; sh_live[wave] = live; }
+    __syncthreads();
+    first = min(min(sh_first[0], sh_first[1]), min(sh_first[2], sh_first[3]));
+    live = max(max(sh_live[0], sh_live[1]), max(sh_live[2], sh_live[3]));
+    const int owner = first != 0x7fffffff ? first : live;
+    if (owner < 0) {                                     // every weight of the chunk underflowed: its first column
+        if (threadIdx.x == 0) out_tokens[b] = min(chunk * kCdfChunk, vocab - 1);
+        return;
+    }
+    if (static_cast<int>(threadIdx.x) == owner) {
+        float run = incl - mine;
+        int tok = -1, last = c0;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            if (w[j] > 0.f) last = c0 + j;
+            if (tok < 0 && w[j] > 0.f && run + w[j] > rest) tok = c0 + j;
+            run += w[j];
+        }
+        out_tokens[b] = tok < 0 ? last : tok;
     }
 }
 
@@ -326,12 +494,13 @@ extern "C" int nva_sample(const void *logits, int64_t logits_row_stride, const f
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bf16_t *lg = static_cast<const bf16_t *>(logits);
     if (noise == nullptr) {
-        const int gchunks = gumbel_chunks(vocab);              // fewer, wider chunks: fits the same workspace
-        hipLaunchKernelGGL(sampler_gumbel_kernel, dim3(gchunks, batch), dim3(kSampThreads), 0, s, lg,
-                           logits_row_stride, temperatures, seed, offset, part_best, part_idx, vocab, gchunks);
+        const int cchunks = cdf_chunks(vocab);                 // fewer, wider chunks: fits the same workspace
+        hipLaunchKernelGGL(sampler_cdf_sums_kernel, dim3(cchunks, batch), dim3(kSampThreads), 0, s, lg,
+                           logits_row_stride, temperatures, part_max, part_sum, part_best, part_idx, vocab, cchunks);
         if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL(sampler_pick_kernel, dim3(batch), dim3(kWave), 0, s, part_best, part_idx, out_tokens,
-                           gchunks);
+        hipLaunchKernelGGL(sampler_cdf_select_kernel, dim3(batch), dim3(kSampThreads), 0, s, lg, logits_row_stride,
+                           temperatures, seed, offset, part_max, part_sum, part_best, part_idx, out_tokens, vocab,
+                           cchunks);
         return launch_status();
     }
     hipLaunchKernelGGL(sampler_partials_kernel, dim3(nchunks, batch), dim3(kSampThreads), 0, s, lg,

@@ -19,7 +19,8 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor, noise: Optional[tor
     """``argmax(softmax(logits.float() / T) / clamp_min(E, 1e-10))`` per row.
 
     ``noise`` (fp32 ``[B, V]``) supplies ``E`` explicitly so a draw can be replayed; with
-    ``noise=None`` the kernel draws ``E`` itself from Philox keyed by ``(seed, offset)``.
+    ``noise=None`` the kernel draws the token from the same categorical distribution by inverse
+    CDF with one Philox uniform per row keyed by ``(seed, offset)``.
     Rows with temperature 0 return ``argmax(logits)``.
     """
     assert logits.dim() == 2 and logits.dtype == torch.bfloat16 and logits.stride(1) == 1
@@ -49,7 +50,7 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor, noise: Optional[tor
 class Sampler(nn.Module):
     """``forward(logits, temperatures)`` as in nanovllm/layers/sampler.py:10-15.
 
-    Each call advances a Philox offset, so successive calls draw fresh noise while a run
+    Each call advances a Philox offset, so successive calls draw afresh while a run
     with the same ``seed`` is reproducible.
     """
 

@@ -14,6 +14,10 @@ here: GQA mapping ``h_kv = h_q // (Hq // Hkv)``, paged layout ``[num_blocks, pag
 bottom-right aligned causal mask when ``seqlen_k > seqlen_q`` (flash-attn >= 2.1), fp32
 softmax/accumulation and zero output for rows that see no keys.
 
+For draws without a noise tensor the library's own scheme is restated as well: one Philox4x32-10
+uniform per row (``philox4x32_10``, ``row_uniforms``; pinned by the Random123 known-answer vectors)
+walked through float64 running sums of the softmax (``inverse_cdf_bounds``).
+
 Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
 import this package, and only as the checker / the timed CPU baseline.  Nothing under the
 product package imports it; the product fails loudly when its HIP library is missing.
@@ -28,6 +32,9 @@ from .hotpath import (  # noqa: F401
     gather_pages,
     paged_decode_attention,
     varlen_prefill_attention,
+    philox4x32_10,
+    row_uniforms,
+    inverse_cdf_bounds,
     sample,
     sample_scores,
 )

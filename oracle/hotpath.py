@@ -192,3 +192,39 @@ def sample(logits, temperatures, noise):
     if bool(greedy.any()):
         tokens = torch.where(greedy, logits.float().argmax(dim=-1), tokens)
     return tokens
+
+
+# ------------------------------------------------------------------ draws without a noise tensor
+def philox4x32_10(counter, key):
+    """Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3",
+    SC'11): ``counter`` four and ``key`` two 32-bit words; returns the four output words.
+    Pinned by the known-answer vectors of the authors' Random123 distribution."""
+    m0, m1, w0, w1 = 0xD2511F53, 0xCD9E8D57, 0x9E3779B9, 0xBB67AE85
+    c = [int(x) & 0xFFFFFFFF for x in counter]
+    k = [int(x) & 0xFFFFFFFF for x in key]
+    for _ in range(10):
+        p0, p1 = m0 * c[0], m1 * c[2]
+        c = [(p1 >> 32) ^ c[1] ^ k[0], p1 & 0xFFFFFFFF, (p0 >> 32) ^ c[3] ^ k[1], p0 & 0xFFFFFFFF]
+        k = [(k[0] + w0) & 0xFFFFFFFF, (k[1] + w1) & 0xFFFFFFFF]
+    return c
+
+
+def row_uniforms(seed, offset, batch):
+    """The uniform in (0, 1) that the library draws for row ``b`` of a call keyed by
+    ``(seed, offset)`` when no noise tensor is given: first output word of Philox4x32-10 with
+    counter ``(b, 0x5a17, offset_lo, offset_hi)`` and key ``(seed_lo, seed_hi)``; its top 24 bits
+    plus one half, times 2**-24.  float64 ``[batch]``."""
+    out = torch.empty(batch, dtype=torch.float64)
+    for b in range(batch):
+        r = philox4x32_10((b, 0x5A17, offset & 0xFFFFFFFF, (offset >> 32) & 0xFFFFFFFF),
+                          (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))
+        out[b] = ((r[0] >> 8) + 0.5) * 2.0 ** -24
+    return out
+
+
+def inverse_cdf_bounds(logits, temperatures):
+    """float64 running sums of ``softmax(logits / T)`` per row, ``[B, V]``: the token drawn for a
+    uniform ``u`` is the first column whose running sum exceeds ``u`` -- a draw from the same
+    categorical distribution as the exponential race of nanovllm/layers/sampler.py:12-14."""
+    p = torch.softmax(logits.double() / temperatures.double().unsqueeze(1), dim=-1)
+    return p.cumsum(-1)

@@ -93,6 +93,30 @@ def test_sampler_philox_mode_is_categorical_and_reproducible(dev):
     assert x.shape == (n,) and not torch.equal(x, y)
 
 
+@pytest.mark.parametrize("batch,vocab,scale", [(64, 151936, 2.0), (33, 4001, 1.0), (8, 50000, 4.0), (5, 7, 1.0)])
+def test_sampler_in_kernel_draw_is_the_inverse_cdf_of_its_uniform(dev, batch, vocab, scale):
+    """Without a noise tensor the token of row b is the first column whose running sum of
+    softmax(logits / T) exceeds u_b, with u_b the Philox uniform of (seed, offset, b).  The kernel
+    sums in fp32 and in chunks, so the float64 running sums of the oracle must bracket u_b to
+    within that rounding, and most rows agree exactly."""
+    g = torch.Generator().manual_seed(vocab)
+    logits = (torch.randn(batch, vocab, generator=g) * scale).to(torch.bfloat16)
+    logits[0, : min(3, vocab - 1)] = float("-inf")           # leading columns that cannot be drawn
+    temps = torch.linspace(0.5, 1.3, batch)
+    seed, offset = 0x1234567811, 77
+    tok = sample(logits.to(dev), temps.to(dev), None, seed=seed, offset=offset).cpu()
+    u = oracle.row_uniforms(seed, offset, batch)
+    bounds = oracle.inverse_cdf_bounds(logits, temps)
+    rows = torch.arange(batch)
+    hi = bounds[rows, tok]
+    lo = torch.where(tok > 0, bounds[rows, (tok - 1).clamp_min(0)], torch.zeros(batch, dtype=torch.float64))
+    tol = 2e-5
+    assert bool(((lo - tol <= u) & (u <= hi + tol)).all()), (u, lo, hi)
+    assert bool((hi > lo).all())                               # never a column of zero probability
+    want = torch.searchsorted(bounds, u.unsqueeze(1), right=True).squeeze(1).clamp_max(vocab - 1)
+    assert float((tok == want).double().mean()) >= 0.9
+
+
 def test_sampler_philox_mode_large_vocab_and_greedy(dev):
     """In-kernel noise on a wide, flat vocabulary: bucketed chi-square against the softmax, a
     dominant logit always wins, and temperature-0 rows are plain argmax."""

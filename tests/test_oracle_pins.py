@@ -313,3 +313,31 @@ def test_sampler_is_a_categorical_draw():
     p = torch.softmax(logits.double()[0] / t, -1)
     chi2 = float(((freq - n * p) ** 2 / (n * p)).sum())
     assert chi2 < 40.0     # 11 dof: P(chi2 > 40) ~ 4e-5
+
+
+# ------------------------------------------------------------------ draws without a noise tensor
+def test_philox_known_answers():
+    """Known-answer vectors of Philox4x32-10 from the authors' Random123 distribution
+    (kat_vectors: counter words, key words -> output words)."""
+    assert oracle.philox4x32_10((0, 0, 0, 0), (0, 0)) == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    assert oracle.philox4x32_10((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2) == [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]
+    assert oracle.philox4x32_10((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0)) == [
+        0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]
+    u = oracle.row_uniforms(seed=7, offset=3, batch=2000)
+    assert float(u.min()) > 0 and float(u.max()) < 1
+    assert abs(float(u.mean()) - 0.5) < 0.03 and not torch.equal(u, oracle.row_uniforms(7, 4, 2000))
+
+
+def test_inverse_cdf_draws_the_softmax():
+    """Walking the running sums with an even grid of uniforms reproduces every probability to
+    within one grid step: the draw is categorical in softmax(logits / T), like the race."""
+    row = torch.tensor([[2.0, 1.0, 0.5, 0.0, -0.5, -1.0, 1.5, 0.25]]).to(torch.bfloat16)
+    t = torch.tensor([0.7])
+    bounds = oracle.inverse_cdf_bounds(row, t)[0]
+    assert abs(float(bounds[-1]) - 1.0) < 1e-12 and bool((bounds[1:] >= bounds[:-1]).all())
+    n = 100000
+    u = (torch.arange(n, dtype=torch.float64) + 0.5) / n
+    tok = torch.searchsorted(bounds, u, right=True).clamp_max(row.shape[1] - 1)
+    freq = torch.bincount(tok, minlength=row.shape[1]).double() / n
+    p = torch.softmax(row[0].double() / 0.7, -1)
+    assert float((freq - p).abs().max()) <= 1.0 / n + 1e-12
