@@ -11,6 +11,10 @@
 // whatever the mix of context lengths, nothing is launched for empty table entries, and
 // the 8 XCDs (which receive workgroups round-robin) stay balanced.  The grid depends on no
 // device data, so the launch can be captured in a HIP graph and replayed with new contents.
+// The split (prefix sums, clipped lengths, first stage and slice of every worker) is left in the
+// workspace; a later launch over the same context_lens and block_tables -- the next layer of the
+// same decode step -- may start from it (decode_stream_kernel<G, true>) and then issues its first
+// loads after one 32-byte read instead of three dependent memory round trips.
 //
 // Per worker, a two-deep software pipeline over its stages:
 //   * HBM -> VGPR: a K (or V) head row is 128 bf16 = 256 B = 16 lanes x 16 B, so one dwordx4
@@ -36,7 +40,8 @@
 // the whole kernel.  Relaxed device-scope atomics without fences returned stale partials.)
 //
 // HBM traffic per sequence and layer: ctx * num_kv_heads * 128 * 2 B for K plus the same for
-// V (4096 B per token at 8 kv heads).  Partials: at most (W + batch*num_kv_heads) * G rows of 520 B.
+// V (4096 B per token at 8 kv heads).  Partials: at most (W + batch*num_kv_heads) * G rows of 520 B;
+// the stored split: 64 KB of worker records and 8 bytes per sequence.
 #include "nva_common.h"
 
 #include <math.h>
