@@ -335,55 +335,61 @@ __global__ __launch_bounds__(kSampThreads) void sampler_cdf_select_kernel(
         return;
     }
     const float k = 1.4426950408889634f / t_in;
-    // ---- row maximum and the chunk weights relative to it -------------------------------------
-    float m = -INFINITY;
-    for (int c = threadIdx.x; c < nchunks; c += kSampThreads)
-        m = fmaxf(m, part_max[static_cast<int64_t>(b) * nchunks + c]);
-    m = block_max4(m, sh, lane, wave);
-    if (m == -INFINITY) {                                // no finite logit in the row
-        if (threadIdx.x == 0) out_tokens[b] = 0;
-        return;
-    }
-    // one uniform per row, in (0, 1): 24 random bits plus one half
-    const uint2 key = make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
-    const uint4 r = Philox::draw(make_uint4(static_cast<uint32_t>(b), 0x5a17u, static_cast<uint32_t>(offset),
-                                            static_cast<uint32_t>(offset >> 32)), key);
-    const float u = (static_cast<float>(r.x >> 8) + 0.5f) * 5.9604644775390625e-8f;
-    // chunk weights into LDS (all lanes), then one lane walks them: running sum in chunk order
-    constexpr int kLdsChunks = 1024;                     // rows with more chunks walk the workspace instead
-    __shared__ float sh_w[kLdsChunks];
-    const bool in_lds = nchunks <= kLdsChunks;
-    if (in_lds)
-        for (int c = threadIdx.x; c < nchunks; c += kSampThreads) {
-            const int64_t at = static_cast<int64_t>(b) * nchunks + c;
-            sh_w[c] = part_sum[at] * __builtin_amdgcn_exp2f(part_max[at] - m);
+    // ---- wavefront 0: row maximum, chunk weights relative to it, and the chunk that holds u * total ----
+    if (wave == 0) {
+        const float *pm = part_max + static_cast<int64_t>(b) * nchunks;
+        const float *ps = part_sum + static_cast<int64_t>(b) * nchunks;
+        float m = -INFINITY;
+        for (int c = lane; c < nchunks; c += kWave) m = fmaxf(m, pm[c]);
+        m = wave_max(m);
+        int pick = -2;                                   // -2: no finite logit in the row
+        float rest_in_chunk = 0.f;
+        if (m != -INFINITY) {
+            float total = 0.f;
+            for (int c = lane; c < nchunks; c += kWave) total += ps[c] * __builtin_amdgcn_exp2f(pm[c] - m);
+            total = wave_sum(total);
+            // one uniform per row, in (0, 1): 24 random bits plus one half
+            const uint2 key = make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+            const uint4 r = Philox::draw(make_uint4(static_cast<uint32_t>(b), 0x5a17u, static_cast<uint32_t>(offset),
+                                                    static_cast<uint32_t>(offset >> 32)), key);
+            const float u = (static_cast<float>(r.x >> 8) + 0.5f) * 5.9604644775390625e-8f;
+            const float target = u * total;
+            // running sum in chunk order, 64 chunks at a time
+            float carry = 0.f;
+            int last_live = 0;
+            pick = -1;
+            for (int base = 0; base < nchunks; base += kWave) {
+                const int c = base + lane;
+                const float w = c < nchunks ? ps[c] * __builtin_amdgcn_exp2f(pm[c] - m) : 0.f;
+                float incl = w;
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const float up = __shfl_up(incl, off, 64);
+                    if (lane >= off) incl += up;
+                }
+                incl += carry;
+                const uint64_t live = __builtin_amdgcn_ballot_w64(w > 0.f);
+                const uint64_t hit = __builtin_amdgcn_ballot_w64(w > 0.f && incl > target);
+                if (live != 0) last_live = base + 63 - __builtin_clzll(live);
+                if (pick < 0 && hit != 0) {
+                    const int l = __builtin_ctzll(hit);
+                    pick = base + l;
+                    rest_in_chunk = target - __shfl(incl - w, l, 64);     // what is left to walk inside the chunk
+                }
+                carry = __shfl(incl, 63, 64);
+            }
+            if (pick < 0) { pick = last_live; rest_in_chunk = INFINITY; }   // rounding: beyond the last running sum
         }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        auto weight = [&](int c) {
-            const int64_t at = static_cast<int64_t>(b) * nchunks + c;
-            return in_lds ? sh_w[c] : part_sum[at] * __builtin_amdgcn_exp2f(part_max[at] - m);
-        };
-        float total = 0.f;
-        for (int c = 0; c < nchunks; ++c) total += weight(c);
-        const float target = u * total;
-        float run = 0.f, before = 0.f;
-        int pick = -1, last_live = 0;
-        for (int c = 0; c < nchunks; ++c) {
-            const float w = weight(c);
-            if (w > 0.f) last_live = c;
-            if (pick < 0 && w > 0.f && run + w > target) { pick = c; before = run; }
-            run += w;
-        }
-        float rest_in_chunk = target - before;                   // what is left to walk inside the chunk
-        if (pick < 0) { pick = last_live; rest_in_chunk = INFINITY; }   // rounding: beyond the last running sum
-        sh_pick[0] = pick;
-        sh[0] = rest_in_chunk;
+        if (lane == 0) { sh_pick[0] = pick; sh[0] = rest_in_chunk; sh[1] = m; }
     }
     __syncthreads();
     const int chunk = sh_pick[0];
     const float rest = sh[0];
-    __syncthreads();
+    const float m = sh[1];
+    if (chunk == -2) {
+        if (threadIdx.x == 0) out_tokens[b] = 0;
+        return;
+    }
     // ---- inside the chunk: 32 consecutive columns per lane, scan over the 256 lanes -------------
     const bf16_t *row = logits + static_cast<int64_t>(b) * row_stride;
     const int c0 = chunk * kCdfChunk + threadIdx.x * 32;
