@@ -11,7 +11,8 @@ already resident in HBM.  Workloads (shapes are the five benchmark configuration
     scatter   store_kvcache, 4096 tokens into 512 blocks x 256 slots              (config 1)
     prefill   causal varlen prefill, 16 sequences, half with cached prefix        (config 3)
     sampler   temperature sampling over 256 x 151,936 logits
-    decode-e2e-shape / copy   profiling helpers: the roofline leg of e2e alone; a plain copy of known size
+    decode-e2e-shape / decode-longctx-shape / copy   profiling helpers: the decode attention of configs 4 / 5
+              alone (one layer); a plain copy of known size
 The line carries `roofline` (algorithmic bytes or flops of the dominant kernel per launch,
 divided by its average duration measured with HIP events on the launch stream) and
 `cpu_baseline` (the CPU oracle timed on this box's host cores on a bounded sample).
