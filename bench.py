@@ -15,7 +15,11 @@ already resident in HBM.  Workloads (shapes are the five benchmark configuration
               alone (one layer); a plain copy of known size
 The line carries `roofline` (algorithmic bytes or flops of the dominant kernel per launch,
 divided by its average duration measured with HIP events on the launch stream) and
-`cpu_baseline` (the CPU oracle timed on this box's host cores on a bounded sample).
+`cpu_baseline` (the CPU oracle timed on this box's host cores on a bounded sample).  The default
+(e2e) line also carries `extra`: the rooflines of the scatter, decode, prefill and sampler
+configurations and of the long-context decode shape, each timed in isolation in the same run, and
+one eager (no hipGraph) pass of the same workload.  Every timed e2e pass generates from prompts
+the engine has not seen (fresh draw per pass), like the reference's bench.py:22-27.
 Only one GPU is used; --gpus above 1 is refused.
 """
 import argparse
@@ -50,6 +54,13 @@ def _event_time_ms(fn_list, steps, warmup):
     return start.elapsed_time(stop)
 
 
+def _cpu_cores():
+    """Threads the CPU baseline really runs on (torch's intra-op pool, which follows OMP_NUM_THREADS),
+    and what the host reports."""
+    import torch
+    return {"cores": torch.get_num_threads(), "host_cpu_count": os.cpu_count()}
+
+
 def _median_cpu_seconds(fn, repeats=5, warm=1):
     for _ in range(warm):
         fn()
@@ -63,47 +74,39 @@ def _median_cpu_seconds(fn, repeats=5, warm=1):
 
 # ----------------------------------------------------------------------------- workloads
 def bench_decode(args, dev):
+    """Config 2.  Timed the way an engine calls it: 28 launches (the layers of one decode step of
+    Qwen3-0.6B) share one work split, each on the KV pool of its own "layer" (4 rotating 1 GiB
+    pools, so the 256 MB Infinity Cache cannot serve re-reads).  `standalone_us_per_launch` is the
+    same call without a shared split (every launch derives it)."""
     import torch
-    import nanovllm_amd as nva
     from nanovllm_amd import synthetic
-    pools = 4                      # rotate 1 GiB pools so the 256 MB Infinity Cache cannot serve re-reads
-    cases, fns, alg = [], [], []
+    pools = 4
+    caches = []
     for p in range(pools):
         g = torch.Generator(device=dev).manual_seed(100 + p)
-        kc = torch.randn((1024, 256, 8, 128), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
-        vc = torch.randn((1024, 256, 8, 128), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
-        c = synthetic.decode_case(seed=p, cache=(kc, vc))
-        q, cl, bt = c.q.to(dev), c.context_lens.to(dev), c.block_tables.to(dev)
-        out = torch.empty((64, 1, 16, 128), dtype=torch.bfloat16, device=dev)
-        cases.append(c)
-        alg.append(c.algorithmic_bytes)
-        fns.append(lambda q=q, kc=kc, vc=vc, cl=cl, bt=bt, s=c.scale, out=out:
-                   nva.paged_decode_attention(q, kc, vc, cl, bt, s, out=out))
-    ms = _event_time_ms(fns, args.steps, args.warmup)
-    per_step_ms = ms / args.steps
-    mean_alg = sum(alg[(args.warmup + i) % pools] for i in range(args.steps)) / args.steps
-    gbps = mean_alg / (per_step_ms * 1e-3) / 1e9
-    tokens = sum(int(c.context_lens.sum()) for c in cases) / pools
+        caches.append(tuple(torch.randn((1024, 256, 8, 128), generator=g, device=dev, dtype=torch.float32)
+                            .to(torch.bfloat16) for _ in range(2)))
+    case = synthetic.decode_case(seed=0, cache=(None, None))      # context lengths only; the tables are drawn per pool
+    ctx = case.context_lens
+    roof = decode_shape_roofline(dev, caches, 1024, ctx, 16, "config 2: batch 64, ctx U[100,2048]", width=8, layers=28,
+                                 steps=args.steps)
+    alone = decode_shape_roofline(dev, caches, 1024, ctx, 16, "", width=8, layers=None, steps=args.steps)
+    roof["standalone_us_per_launch"] = alone["us_per_launch"]
     result = {
         "metric": "paged decode attention, achieved HBM GB/s (config 2)",
-        "value": round(gbps, 1), "unit": "GB/s",
-        "ms_per_step": round(per_step_ms, 5),
+        "value": roof["achieved"], "unit": "GB/s", "ms_per_step": round(roof["us_per_launch"] / 1e3, 5),
         "config": {"workload": "paged_decode_attn config2: batch 64, 16q/8kv heads, head_dim 128, block 256, "
-                               "ctx U[100,2048], 4 rotating 1 GiB KV pools",
-                   "batch": 64, "kv_tokens_per_step": tokens},
-        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "decode_stream_kernel<2> + decode_merge_kernel<2>",
-                     "algorithmic_bytes_per_launch": int(mean_alg)},
+                               "ctx U[100,2048], 4 rotating 1 GiB KV pools, 28 launches per work split",
+                   "batch": 64, "kv_tokens_per_step": int(ctx.sum())},
+        "roofline": roof,
     }
 
     def cpu():
         import oracle
-        c = cases[0]
-        kc, vc = c.k_cache.cpu(), c.v_cache.cpu()
+        c = synthetic.decode_case(seed=0)
         sec = _median_cpu_seconds(lambda: oracle.paged_decode_attention(
-            c.q, kc, vc, c.context_lens, c.block_tables, c.scale, "sdpa"), repeats=5)
-        return {"value": round(alg[0] / sec / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            c.q, c.k_cache, c.v_cache, c.context_lens, c.block_tables, c.scale, "sdpa"), repeats=5)
+        return {"value": round(c.algorithmic_bytes / sec / 1e9, 3), "unit": "GB/s", **_cpu_cores(),
                 "kind": "port", "sample": "config 2 full batch (64 sequences), bf16 torch SDPA on gathered pages, "
                                           "median of 5", "seconds": round(sec, 4)}
     return result, cpu
@@ -139,7 +142,7 @@ def bench_scatter(args, dev):
         c = cases[0]
         sec = _median_cpu_seconds(lambda: oracle.store_kvcache(c.key, c.value, c.k_cache, c.v_cache, c.slot_mapping),
                                   repeats=7)
-        return {"value": round(alg[0] / sec / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+        return {"value": round(alg[0] / sec / 1e9, 3), "unit": "GB/s", **_cpu_cores(),
                 "kind": "port", "sample": "config 1 full size, torch index_copy_, median of 7",
                 "seconds": round(sec, 5)}
     return result, cpu
@@ -175,7 +178,7 @@ def bench_prefill(args, dev):
         oracle.store_kvcache(c.k, c.v, ek, ev, c.slot_mapping)
         sec = _median_cpu_seconds(lambda: oracle.varlen_prefill_attention(
             c.q, None, None, c.cu_seqlens_q, c.cu_seqlens_k, c.scale, ek, ev, c.block_tables, "sdpa"), repeats=3)
-        return {"value": round(flops / sec / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+        return {"value": round(flops / sec / 1e12, 4), "unit": "TFLOP/s", **_cpu_cores(),
                 "kind": "port", "sample": "config 3 full batch, bf16 torch SDPA with explicit lower-right mask, "
                                           "median of 3", "seconds": round(sec, 3)}
     return result, cpu
@@ -213,7 +216,7 @@ def bench_sampler(args, dev):
         t = temps[:64].cpu()
         noise = torch.empty(64, vocab).exponential_(1.0)
         sec = _median_cpu_seconds(lambda: oracle.sample(l, t, noise), repeats=5)
-        return {"value": round(64 * vocab * 2 / sec / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+        return {"value": round(64 * vocab * 2 / sec / 1e9, 3), "unit": "GB/s", **_cpu_cores(),
                 "kind": "port", "sample": "64 of the 256 rows, eager torch sampler with pre-drawn noise, "
                                           "median of 5", "seconds": round(sec, 4)}
     return result, cpu
@@ -230,13 +233,23 @@ def e2e_workload(num_seqs=256, max_input_len=1024, max_output_len=1024, vocab=15
     return prompts, params
 
 
-# HBM bytes per launch of decode_stream_kernel<2> at the e2e decode shape, from two rocprofv3 --pmc
-# passes of `bench.py --workload decode-e2e-shape` (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each
-# scaled by what the same counter reads for the plain copy kernel of `--workload copy` (known size).
-MEASURED_TRAFFIC_E2E_SHAPE = 863_700_000      # stream kernel 858.8 MB + merge kernel 4.9 MB (algorithmic: 855.3 MB)
+TRAFFIC_PROFILE = "profiles/hbm_traffic_pmc__all_kernels.txt"
 
 
-def decode_shape_roofline(dev, caches, num_blocks, ctx, hq, what, traffic=None, width=None, layers=None):
+def measured_traffic(key):
+    """HBM bytes per launch from the tracked summary of the two rocprofv3 --pmc passes (FETCH_SIZE, then
+    WRITE_SIZE, each scaled by what the same counter reads for the plain copy of `--workload copy`):
+    the line `traffic_bytes_per_launch[<key>] = <bytes>` of TRAFFIC_PROFILE; None when it is absent."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic_bytes_per_launch\[%s\]\s*=\s*([0-9_]+)" % re.escape(key), text)
+    return int(m.group(1).replace("_", "")) if m else None
+
+
+def decode_shape_roofline(dev, caches, num_blocks, ctx, hq, what, traffic=None, width=None, layers=None, steps=None):
     """Paged decode attention for the context lengths ``ctx``: block tables drawn without
     replacement from the pool, timed with HIP events while rotating through `caches` (separate
     K/V pools, so neither L2 nor the 256 MB Infinity Cache can serve re-reads).  With ``layers``
@@ -265,6 +278,8 @@ def decode_shape_roofline(dev, caches, num_blocks, ctx, hq, what, traffic=None, 
 
     fns = [lambda kc=kc, vc=vc: call(kc, vc) for kc, vc in caches]
     reps = 3 * layers if layers else max(5 * len(fns), 60)      # whole steps: one build per `layers` calls
+    if steps and steps > 1:
+        reps = -(-steps // layers) * layers if layers else steps
     ms = _event_time_ms(fns, reps, layers if layers else len(fns)) / reps
     alg = int(ctx.sum()) * hkv * dh * 2 * 2 + 2 * q.numel() * 2
     gbps = alg / (ms * 1e-3) / 1e9
@@ -282,9 +297,11 @@ def decode_e2e_shape_roofline(dev, caches, num_blocks):
     import torch
     prompts, params = e2e_workload()
     ctx = torch.tensor([len(p) + sp.max_tokens // 2 for p, sp in zip(prompts, params)], dtype=torch.int32)
-    return decode_shape_roofline(dev, caches, num_blocks, ctx, 16, "batch 256", MEASURED_TRAFFIC_E2E_SHAPE,
+    roof = decode_shape_roofline(dev, caches, num_blocks, ctx, 16, "batch 256", measured_traffic("decode_e2e_shape"),
                                  width=16,           # the engine's static table width at max_model_len 4096
                                  layers=28)          # Qwen3-0.6B
+    roof["traffic_source"] = TRAFFIC_PROFILE
+    return roof
 
 
 def bench_decode_longctx_shape(args, dev):
@@ -341,8 +358,63 @@ def bench_copy(args, dev):
     return result, (lambda: None)
 
 
+def fresh_prompts(prompts, pass_index, vocab=151936):
+    """Prompts of the same lengths with newly drawn token ids: every timed pass must prefill prompts
+    the engine has never seen (its prefix cache keeps the hashes of freed blocks), as the reference's
+    single timed generate() does (bench.py:22-27)."""
+    import random
+    rng = random.Random(10_000 + pass_index)
+    return [[rng.randint(0, vocab - 1) for _ in p] for p in prompts]
+
+
+def _e2e_passes(llm, prompts, params, passes, first_pass):
+    """Time `passes` generate() calls, each on freshly drawn prompt ids; returns seconds."""
+    import torch
+    for k in llm.stats:
+        llm.stats[k] = 0
+    batches = [fresh_prompts(prompts, first_pass + i) for i in range(passes)]      # drawn outside the timed region
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for batch in batches:
+        outs = llm.generate(batch, params)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert all(len(o["token_ids"]) == p.max_tokens for o, p in zip(outs, params))
+    return dt
+
+
+def collect_extra(dev, model, prompts, params):
+    """The other configurations, each timed in isolation (a second or less of GPU time each), and one
+    eager pass of the e2e workload, for the `extra` object of the default line."""
+    import gc
+    import torch
+    from types import SimpleNamespace
+    from nanovllm_amd.engine.llm import LLM
+    extra = {}
+    for name, fn, steps in (("scatter_config1", bench_scatter, 400), ("decode_config2", bench_decode, 112),
+                            ("prefill_config3", bench_prefill, 50), ("sampler_256x151936", bench_sampler, 100),
+                            ("decode_config5_shape", bench_decode_longctx_shape, 1)):
+        result, _ = fn(SimpleNamespace(steps=steps, warmup=max(3, steps // 10)), dev)
+        extra[name] = dict(result["roofline"], us_per_launch=round(result["ms_per_step"] * 1e3, 2))
+        del result
+        gc.collect()
+        torch.cuda.empty_cache()
+    llm = LLM(model, enforce_eager=True, max_model_len=4096, num_kvcache_blocks=4096)
+    llm.generate(fresh_prompts(prompts[:32], 9_000), params[:32])
+    dt = _e2e_passes(llm, prompts, params, 1, 5_000)
+    total_out = sum(p.max_tokens for p in params)
+    extra["e2e_eager"] = {"value": round(total_out / dt, 1), "unit": "tok/s", "s_per_pass": round(dt, 3),
+                          "what": "the same 256-request workload with enforce_eager=True (no hipGraph decode), one pass",
+                          "prefill_s": round(llm.stats["prefill_s"], 3), "decode_s": round(llm.stats["decode_s"], 3)}
+    del llm
+    gc.collect()
+    torch.cuda.empty_cache()
+    return extra
+
+
 def bench_e2e(args, dev):
     """Qwen3-0.6B architecture, random weights, 256 requests, hipGraph decode: output tok/s."""
+    import gc
     import torch
     import nanovllm_amd as nva
     from nanovllm_amd.engine import SamplingParams, qwen3_0_6b
@@ -352,36 +424,41 @@ def bench_e2e(args, dev):
     prompts, params = e2e_workload(num_seqs=args.requests, max_output_len=args.max_output_len)
     total_out = sum(p.max_tokens for p in params)
     llm.generate([[1, 2, 3, 4]], SamplingParams(max_tokens=8, ignore_eos=True))     # reference warm-up call
-    for _ in range(args.warmup):
-        llm.generate(prompts[:32], params[:32])
-    for k in llm.stats:
-        llm.stats[k] = 0
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        outs = llm.generate(prompts, params)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    assert all(len(o["token_ids"]) == p.max_tokens for o, p in zip(outs, params))
+    for w in range(args.warmup):
+        llm.generate(fresh_prompts(prompts[:32], 9_000 + w), params[:32])
+    dt = _e2e_passes(llm, prompts, params, args.steps, 0)
     tok_s = total_out * args.steps / dt
 
     layers = [m for m in llm.model_runner.model.modules() if isinstance(m, nva.Attention)]
     roof = decode_e2e_shape_roofline(dev, [(a.k_cache, a.v_cache) for a in layers], llm.config.num_kvcache_blocks)
-    st = llm.stats
+    st = dict(llm.stats)
+    del layers, llm
+    gc.collect()
+    torch.cuda.empty_cache()
     result = {
         "metric": "output tok/s, Qwen3-0.6B bench shape; decode-attn HBM GB/s vs ~8 TB/s",
         "value": round(tok_s, 1), "unit": "tok/s", "ms_per_step": round(dt / args.steps * 1e3, 2),
         "config": {"workload": "e2e generate: Qwen3-0.6B architecture (28 layers, hidden 1024, 16q/8kv heads x 128, "
                                "MLP 3072, vocab 151936, random bf16 weights), 256 requests, prompt and output lengths "
-                               "U[100,1024], temperature 0.6, ignore_eos, " + ("eager" if args.eager else "hipGraph decode"),
-                   "requests": 256, "output_tokens": total_out, "engine_steps_per_pass": (st["prefill_steps"] + st["decode_steps"]) // args.steps,
+                               "U[100,1024], temperature 0.6, ignore_eos, prompt ids drawn afresh for every pass, "
+                               + ("eager" if args.eager else "hipGraph decode"),
+                   "requests": args.requests, "output_tokens": total_out, "engine_steps_per_pass": (st["prefill_steps"] + st["decode_steps"]) // args.steps,
                    "prefill_s_per_pass": round(st["prefill_s"] / args.steps, 3), "decode_s_per_pass": round(st["decode_s"] / args.steps, 3)},
         "roofline": roof,
     }
+    if not args.no_extra:
+        result["extra"] = collect_extra(dev, model, prompts, params)
 
     def cpu():
         from oracle import engine_cpu
-        return engine_cpu.baseline(model, prompts, params)
+        # the same mix at one eighth of the lengths (prompt and output alike, so the share of prefill
+        # and decode work is the workload's), first 16 requests: what the host finishes in ~20 s
+        short = [p[: max(1, len(p) // 8)] for p in prompts[:16]]
+        sp = [SamplingParams(temperature=q.temperature, ignore_eos=True, max_tokens=max(1, q.max_tokens // 8)) for q in params[:16]]
+        base = engine_cpu.baseline(model, short, sp, num_requests=16, max_new_tokens=1 << 30, budget_s=40.0)
+        base["sample"] = "prompt and output lengths of the bench mix divided by 8: " + base["sample"]
+        base.update(_cpu_cores())
+        return base
     return result, cpu
 
 
@@ -481,6 +558,7 @@ def main():
     ap.add_argument("--requests", type=int, default=256, help="e2e only: number of requests (profiling runs)")
     ap.add_argument("--max-output-len", type=int, default=1024, help="e2e only: cap on output lengths (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="e2e only: skip the per-configuration rooflines and the eager pass")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the hot path needs no collectives); "
@@ -493,7 +571,6 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible (the hot path has no CPU fallback)")
-    torch.set_num_threads(min(os.cpu_count() or 1, 16))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     from nanovllm_amd import _lib
@@ -506,6 +583,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic", "config": result["config"], "roofline": result["roofline"],
     }
+    if "extra" in result:
+        line["extra"] = result["extra"]
     if not args.no_cpu_baseline:
         base = cpu_fn()
         if base is not None:

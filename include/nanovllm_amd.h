@@ -157,10 +157,14 @@ int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride,
  * temperatures: fp32 [batch].  T == 0 selects greedy argmax(logits) for that row (an
  * extension; the reference forbids T <= 1e-10, nanovllm/sampling_params.py:11).
  * noise: fp32 [batch, vocab] Exp(1) draws (row stride noise_row_stride): the formula above is
- * evaluated as written and a draw can be replayed.  NULL: the token is drawn from the same
- * categorical distribution softmax(logits / T) by inverse CDF (first column whose running sum of
- * probabilities exceeds u), with one uniform u per row from Philox4x32-10 keyed by
- * (seed, offset, row); the same (seed, offset) reproduces the draw.
+ * evaluated (scores relative to the maximum of each 8192-column chunk, rescaled to the row) and a
+ * draw can be replayed; the argmax differs from the formula only between scores that agree to fp32
+ * rounding.  NULL: the token is drawn from the same categorical distribution softmax(logits / T) by a
+ * tree of inverse-CDF steps over the columns in column order (row -> chunk of 8192 -> slice of 2048
+ * -> group of 512 -> group of 8 -> column; at every level the first branch whose running sum of
+ * weights exceeds u * total), each level with its own 32-bit uniform from Philox4x32-10 keyed by
+ * (seed, offset, row, chunk); the same (seed, offset) reproduces the draw.  Sums are fp32 and a
+ * conditional probability below 2^-32 at a level is not resolved.
  * out_tokens: int64 [batch].
  * workspace: at least nva_sample_workspace_bytes() bytes, 16-byte aligned.
  */

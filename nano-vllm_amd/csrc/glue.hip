@@ -96,24 +96,29 @@ static void launch_rms_norm(hipStream_t stream, const bf16_t *x, int64_t x_strid
                            out, residual_out, rows, hidden, eps);
 }
 
-// One wavefront per (token, head) row of 128 elements; lane l holds elements l and l + 64,
-// which are exactly the pair the neox rotation mixes.  Heads [0, hq) are queries, [hq, hq+hkv)
-// keys.  With a cache (k_cache != nullptr) the rotated key row is also written to its cache slot
-// and rows [hq+hkv, hq+2*hkv) copy the value heads to theirs -- the KV scatter fused into the
-// step that produces k (slot -1 or out of range skips the row); without a cache the value rows
-// are not visited at all.
+// Eight lanes per (token, head) row of 128 elements: lane j of a row holds elements [8j, 8j+8) and
+// [64+8j, 64+8j+8) -- the two halves the neox rotation mixes element by element -- so every access
+// to qkv, the weights, the rope table, q_out, k_out and the caches is one 16-byte load or store, and
+// a cache head row of 256 B is written by 8 consecutive lanes (16 for a value row) with dwordx4 stores.  A wavefront covers 8 rows,
+// a workgroup 32.  Heads [0, hq) are queries, [hq, hq+hkv) keys.  With a cache (k_cache != nullptr)
+// the rotated key row is also written to its cache slot and rows [hq+hkv, hq+2*hkv) copy the value
+// heads to theirs -- the KV scatter fused into the step that produces k (slot -1 or out of range
+// skips the row); without a cache the value rows are not visited at all.
 __global__ __launch_bounds__(256) void qk_norm_rope_kernel(
     const bf16_t *__restrict__ qkv, int64_t row_stride, const int64_t *__restrict__ positions,
     const bf16_t *__restrict__ q_weight, const bf16_t *__restrict__ k_weight,
     const float *__restrict__ rope_cache, bf16_t *__restrict__ q_out, bf16_t *__restrict__ k_out,
     bf16_t *__restrict__ k_cache, bf16_t *__restrict__ v_cache, const int32_t *__restrict__ slot_mapping,
     int64_t num_slots, int64_t n_rows, int32_t hq, int32_t hkv, int32_t heads, int32_t max_position, float eps) {
-    const int lane = threadIdx.x & 63;
-    const int64_t r = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-    if (r >= n_rows) return;
+    const int j = threadIdx.x & 7;
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * 32 + (threadIdx.x >> 3);
+    if (r >= n_rows) return;                                             // (whole groups of 8 lanes; the sums below stay inside a group)
     const int64_t tok = r / heads;
     const int head = static_cast<int>(r % heads);
     const bf16_t *src = qkv + tok * row_stride + head * kHeadDim;     // q, k and v heads are adjacent
+    // every load of the row goes out before the first use
+    const u32x4_t lo = *reinterpret_cast<const u32x4_t *>(src + 8 * j);
+    const u32x4_t hi = *reinterpret_cast<const u32x4_t *>(src + 64 + 8 * j);
     int64_t slot = -1;
     if (k_cache != nullptr && head >= hq) {
         slot = slot_mapping[tok];
@@ -122,31 +127,50 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(
     if (head >= hq + hkv) {                                            // value head: cache write only
         if (slot >= 0) {
             bf16_t *dst = v_cache + (slot * hkv + (head - hq - hkv)) * kHeadDim;
-            reinterpret_cast<uint32_t *>(dst)[lane] = reinterpret_cast<const uint32_t *>(src)[lane];
+            *reinterpret_cast<u32x4_t *>(dst + 8 * j) = lo;
+            *reinterpret_cast<u32x4_t *>(dst + 64 + 8 * j) = hi;
         }
         return;
     }
     const bool is_q = head < hq;
     const bf16_t *w = is_q ? q_weight : k_weight;
-    const float x1 = bf16_to_f32(src[lane]);
-    const float x2 = bf16_to_f32(src[lane + 64]);
-    const float ss = wave_sum(fmaf(x1, x1, x2 * x2));
-    const float inv = rsqrtf(ss * (1.0f / kHeadDim) + eps);
-    const float y1 = round_bf16(round_bf16(x1 * inv) * bf16_to_f32(w[lane]));
-    const float y2 = round_bf16(round_bf16(x2 * inv) * bf16_to_f32(w[lane + 64]));
+    const uint4 w1v = *reinterpret_cast<const uint4 *>(w + 8 * j);
+    const uint4 w2v = *reinterpret_cast<const uint4 *>(w + 64 + 8 * j);
     // positions outside the table are clamped instead of read out of bounds
     const int64_t pos = min(max(positions[tok], static_cast<int64_t>(0)), static_cast<int64_t>(max_position) - 1);
-    const float *cs = rope_cache + pos * kHeadDim;
-    const float c = cs[lane], s = cs[lane + 64];
-    const bf16_t o1 = f32_to_bf16(y1 * c - y2 * s);
-    const bf16_t o2 = f32_to_bf16(y2 * c + y1 * s);
+    const float4 *cs = reinterpret_cast<const float4 *>(rope_cache + pos * kHeadDim);
+    const float4 c0 = cs[2 * j], c1 = cs[2 * j + 1], s0 = cs[16 + 2 * j], s1 = cs[16 + 2 * j + 1];
+    const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+    const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+    float x1[8], x2[8], w1[8], w2[8];
+    unpack8(make_uint4(lo[0], lo[1], lo[2], lo[3]), x1);
+    unpack8(make_uint4(hi[0], hi[1], hi[2], hi[3]), x2);
+    unpack8(w1v, w1);
+    unpack8(w2v, w2);
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss = fmaf(x1[i], x1[i], fmaf(x2[i], x2[i], ss));
+    ss += dpp_f32<0xB1>(ss);                                           // sum over the row's 8 lanes: quad_perm [1,0,3,2],
+    ss += dpp_f32<0x4E>(ss);                                           // quad_perm [2,3,0,1],
+    ss += dpp_f32<0x141>(ss);                                          // row_half_mirror
+    const float inv = rsqrtf(ss * (1.0f / kHeadDim) + eps);
+    float o1[8], o2[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float y1 = round_bf16(round_bf16(x1[i] * inv) * w1[i]);
+        const float y2 = round_bf16(round_bf16(x2[i] * inv) * w2[i]);
+        o1[i] = y1 * cv[i] - y2 * sv[i];
+        o2[i] = y2 * cv[i] + y1 * sv[i];
+    }
+    const u32x4_t p1 = {pack_bf16x2(o1[0], o1[1]), pack_bf16x2(o1[2], o1[3]), pack_bf16x2(o1[4], o1[5]), pack_bf16x2(o1[6], o1[7])};
+    const u32x4_t p2 = {pack_bf16x2(o2[0], o2[1]), pack_bf16x2(o2[2], o2[3]), pack_bf16x2(o2[4], o2[5]), pack_bf16x2(o2[6], o2[7])};
     bf16_t *dst = is_q ? q_out + (tok * hq + head) * kHeadDim : k_out + (tok * hkv + (head - hq)) * kHeadDim;
-    dst[lane] = o1;
-    dst[lane + 64] = o2;
+    *reinterpret_cast<u32x4_t *>(dst + 8 * j) = p1;
+    *reinterpret_cast<u32x4_t *>(dst + 64 + 8 * j) = p2;
     if (slot >= 0) {
         bf16_t *cd = k_cache + (slot * hkv + (head - hq)) * kHeadDim;
-        cd[lane] = o1;
-        cd[lane + 64] = o2;
+        *reinterpret_cast<u32x4_t *>(cd + 8 * j) = p1;
+        *reinterpret_cast<u32x4_t *>(cd + 64 + 8 * j) = p2;
     }
 }
 
@@ -244,14 +268,15 @@ extern "C" int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const i
     if (!qkv || !positions || !q_weight || !k_weight || !rope_cache || !q_out || !k_out) return NVA_ERR_NULL_POINTER;
     const bool store = k_cache != nullptr || v_cache != nullptr || slot_mapping != nullptr;
     if (store && (!k_cache || !v_cache || !slot_mapping)) return NVA_ERR_NULL_POINTER;
-    if (qkv_row_stride < static_cast<int64_t>(num_heads + 2 * num_kv_heads) * head_dim || qkv_row_stride % 2 != 0)
+    if (qkv_row_stride < static_cast<int64_t>(num_heads + 2 * num_kv_heads) * head_dim || qkv_row_stride % 8 != 0)
         return NVA_ERR_BAD_STRIDE;
-    if ((reinterpret_cast<uintptr_t>(qkv) & 3u) || (store && ((reinterpret_cast<uintptr_t>(v_cache) & 3u))))
+    if (!aligned16(qkv) || !aligned16(q_weight) || !aligned16(k_weight) || !aligned16(rope_cache) || !aligned16(q_out) ||
+        !aligned16(k_out) || (store && (!aligned16(k_cache) || !aligned16(v_cache))))
         return NVA_ERR_MISALIGNED;
     const int32_t heads = num_heads + (store ? 2 : 1) * num_kv_heads;   // value rows only when they are stored
     const int64_t n_rows = static_cast<int64_t>(n_tokens) * heads;
-    if ((n_rows + 3) / 4 > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;
-    hipLaunchKernelGGL(qk_norm_rope_kernel, dim3(static_cast<uint32_t>((n_rows + 3) / 4)), dim3(256), 0,
+    if ((n_rows + 31) / 32 > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(qk_norm_rope_kernel, dim3(static_cast<uint32_t>((n_rows + 31) / 32)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const bf16_t *>(qkv), qkv_row_stride, positions,
                        static_cast<const bf16_t *>(q_weight), static_cast<const bf16_t *>(k_weight), rope_cache,
                        static_cast<bf16_t *>(q_out), static_cast<bf16_t *>(k_out), static_cast<bf16_t *>(k_cache),

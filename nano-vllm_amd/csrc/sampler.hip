@@ -1,24 +1,38 @@
-// Temperature sampler for gfx950.
+// Temperature sampler for gfx950: one pass over the logits, one tiny merge per row.
 //
 // Replaces Sampler.forward of nanovllm/layers/sampler.py:10-15:
 //     x = float(logits) / T;  p = softmax(x);  token = argmax_i p_i / max(E_i, 1e-10)
-// With a caller-supplied tensor of E ~ Exp(1) draws (replayable; used for parity) the arithmetic
-// keeps the reference's operation order -- true fp32 division by T, exp(x - rowmax) / rowsum, then
-// the division by the clamped noise -- so the argmax can only differ from the reference where two
-// scores are equal to within fp32 rounding.  Without one (what serving uses) the token is drawn
-// from the same categorical distribution by inverse CDF with one in-kernel uniform per row.
 //
-// A row of 151,936 logits is far too little work for one workgroup and 64..256 rows are
-// too few workgroups for 256 CUs, so a row is cut into chunks (one workgroup of 256 lanes each,
-// 16-byte loads of 8 bf16 per lane).
-// With a caller-supplied noise tensor, chunks of 2048 columns:
-//   pass 1  per (chunk, row): chunk max and sum exp(x - chunk max)          -> workspace
-//   pass 2  per (chunk, row): merge the row's partials into (max, sum), then
-//           best p_i / E_i and its column inside the chunk                   -> workspace
-//   pass 3  per row: best chunk, lowest column on ties                       -> int64 token
-// Pass 2 re-reads the logits (2 B/col) that pass 1 pulled through L2 / Infinity Cache.
-// Without noise, chunks of 8192 columns: one pass for the chunk sums, then a per-row selection
-// that re-reads a single chunk (see sampler_cdf_sums_kernel below).
+// A row of 151,936 logits is far too little work for one workgroup and 64..256 rows are too few
+// workgroups for 256 CUs, so a row is cut into chunks of 8192 columns (one workgroup of 256 lanes,
+// four 16-byte loads of 8 bf16 per lane, all issued before the first use, non-temporal: the logits
+// are read exactly once).  sampler_chunk_kernel leaves one 16-byte record per (row, chunk);
+// sampler_row_kernel (one wavefront per row) merges a row's records into the token.
+//
+// With a caller-supplied tensor of E ~ Exp(1) draws (replayable; used for parity) the score of
+// column i is evaluated relative to the CHUNK maximum m_c, e_i = exp(x_i - m_c) / max(E_i, 1e-10)
+// with the reference's true fp32 division by T, and the record keeps (m_c, sum exp, best e_i, its
+// column).  The row merge scales every chunk's best by exp(m_c - M) / S: the same quantity
+// softmax(x)_i / E_i the reference maximises, factored as exp(x_i - m_c) * exp(m_c - M) instead of
+// exp(x_i - M), so the argmax can differ from the reference only where two scores agree to within
+// a few fp32 roundings.  Ties go to the lowest column, as torch.argmax does.
+//
+// Without a noise tensor (what serving uses) there is nothing to replay against, and the token is
+// drawn from the same categorical distribution softmax(x) by a tree of inverse-CDF draws over the
+// columns in column order, every level with a uniform of its own (32 random bits, compared in
+// double precision; a conditional probability below 2^-32 at some level is therefore not
+// resolved, and sums are fp32):
+//     row      -> chunk (8192 columns)   by the chunk weights s_c * exp2(m_c - M)   [row kernel]
+//     chunk    -> slice (2048 columns)   by the four slice sums                     [chunk kernel]
+//     slice    -> wavefront (512)        by the four wavefront sums
+//     wavefront-> lane (8 columns)       by an inclusive scan over the 64 lanes
+//     lane     -> column                 by a walk over its 8 weights
+// The four in-chunk levels run in the chunk kernel on the weights it already holds in registers,
+// so the logits are read once and the row kernel touches only the records.  Uniforms come from
+// Philox4x32-10 keyed by (seed, offset): counter (row, 0x5a17, offset) for the row level, counter
+// (row, 0x10000 + chunk, offset) for the four levels inside a chunk (one output word each).
+// Temperature 0 = greedy argmax of the logits (an extension; nanovllm/sampling_params.py:11
+// forbids it).  A row without any finite logit yields token 0.
 // Algorithmic HBM bytes per row: vocab * 2 B (+ vocab * 4 B when the noise is read).
 #include "nva_common.h"
 
@@ -26,17 +40,32 @@
 
 namespace nva {
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
 constexpr int kSampThreads = 256;
-constexpr int kSampChunk = kSampThreads * 8;   // columns per workgroup
+constexpr int kSampWaves = kSampThreads / kWave;
+constexpr int kSampVec = 4;                               // 16-byte logit loads per lane
+constexpr int kSampSlice = kSampThreads * 8;              // 2048 columns: one load of the whole workgroup
+constexpr int kSampChunk = kSampSlice * kSampVec;         // 8192 columns per workgroup
+constexpr int kNoToken = 0x7fffffff;
 
 __host__ __device__ inline int samp_chunks(int vocab) { return (vocab + kSampChunk - 1) / kSampChunk; }
+
+// One record per (row, chunk), written by the chunk kernel and read by the row kernel.
+//   noise:   {m_c, sum exp(x - m_c), best exp(x - m_c) / max(E, 1e-10), its column}
+//   no noise:{m_c (base 2), sum exp2(y - m_c), unused, the column drawn inside the chunk}
+//   greedy:  {unused, unused, largest logit, its column}
+struct __attribute__((aligned(16))) SampRecord {
+    float m, s, best;
+    int32_t col;
+};
 
 struct Philox {
     // Philox4x32-10 (Salmon et al., SC'11): counter (c0..c3), key (k0,k1)
     __device__ static inline uint4 draw(uint4 c, uint2 k) {
 #pragma unroll
         for (int r = 0; r < 10; ++r) {
-            // one 32x32 -> 64-bit multiply per product (integer multiplies are the slow ops here)
             const uint64_t p0 = static_cast<uint64_t>(0xD2511F53u) * c.x, p1 = static_cast<uint64_t>(0xCD9E8D57u) * c.z;
             const uint32_t hi0 = static_cast<uint32_t>(p0 >> 32), lo0 = static_cast<uint32_t>(p0);
             const uint32_t hi1 = static_cast<uint32_t>(p1 >> 32), lo1 = static_cast<uint32_t>(p1);
@@ -48,434 +77,331 @@ struct Philox {
     }
 };
 
-// Loads the 8 columns [col0, col0+8) of a row as x = float(logit) / T (greedy: T = 1).
-// Columns >= vocab come back as -inf.  vec_ok: the row start is 16-byte aligned.
-__device__ __forceinline__ void load_x8(const bf16_t *row, int col0, int vocab, float temp,
-                                        bool vec_ok, float (&x)[8]) {
-    if (vec_ok && col0 + 8 <= vocab) {
-        const uint4 r = *reinterpret_cast<const uint4 *>(row + col0);
-        unpack8(r, x);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = x[i] / temp;
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            x[i] = (col0 + i < vocab) ? bf16_to_f32(row[col0 + i]) / temp : -INFINITY;
-    }
-}
-
-__global__ __launch_bounds__(kSampThreads) void sampler_partials_kernel(
-    const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
-    float *__restrict__ part_max, float *__restrict__ part_sum, int32_t vocab, int32_t nchunks) {
-    const int chunk = blockIdx.x;
-    const int b = blockIdx.y;
-    const bf16_t *row = logits + static_cast<int64_t>(b) * row_stride;
-    const bool vec_ok = ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
-    float temp = temperatures[b];
-    if (temp == 0.f) temp = 1.f;
-    const int col0 = chunk * kSampChunk + threadIdx.x * 8;
-    float x[8];
-    load_x8(row, col0, vocab, temp, vec_ok, x);
-    float m = x[0];
-#pragma unroll
-    for (int i = 1; i < 8; ++i) m = fmaxf(m, x[i]);
-    m = wave_max(m);
-    __shared__ float sh[4];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (lane == 0) sh[wave] = m;
-    __syncthreads();
-    m = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
-    const float mm = (m == -INFINITY) ? 0.f : m;           // a chunk of -inf logits sums to 0
-    float s = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) s += expf(x[i] - mm);      // exp(-inf) = 0 past the row end
-    s = wave_sum(s);
-    __syncthreads();
-    if (lane == 0) sh[wave] = s;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        part_max[static_cast<int64_t>(b) * nchunks + chunk] = m;
-        part_sum[static_cast<int64_t>(b) * nchunks + chunk] = (sh[0] + sh[1]) + (sh[2] + sh[3]);
-    }
-}
+// 32 random bits -> uniform in (0, 1), exact in double
+__device__ __forceinline__ double unit_uniform(uint32_t r) { return (static_cast<double>(r) + 0.5) * 2.3283064365386963e-10; }
 
 __device__ __forceinline__ void better(float &bs, int &bi, float s, int i) {
     // larger score wins, lower column wins ties (torch.argmax returns the first maximum)
     if (s > bs || (s == bs && i < bi)) { bs = s; bi = i; }
 }
 
-__global__ __launch_bounds__(kSampThreads) void sampler_argmax_kernel(
-    const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
-    const float *__restrict__ noise, int64_t noise_row_stride,
-    const float *__restrict__ part_max, const float *__restrict__ part_sum,
-    float *__restrict__ part_best, int32_t *__restrict__ part_idx, int32_t vocab, int32_t nchunks) {
-    const int chunk = blockIdx.x;
-    const int b = blockIdx.y;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    __shared__ float sh[4];
-    __shared__ int shi[4];
-
-    // row max and row sum from the chunk partials
-    float m = -INFINITY;
-    for (int c = threadIdx.x; c < nchunks; c += kSampThreads)
-        m = fmaxf(m, part_max[static_cast<int64_t>(b) * nchunks + c]);
-    m = wave_max(m);
-    if (lane == 0) sh[wave] = m;
-    __syncthreads();
-    m = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
-    float s = 0.f;
-    for (int c = threadIdx.x; c < nchunks; c += kSampThreads) {
-        const int64_t at = static_cast<int64_t>(b) * nchunks + c;
-        s += part_sum[at] * expf(part_max[at] - m);
-    }
-    s = wave_sum(s);
-    __syncthreads();
-    if (lane == 0) sh[wave] = s;
-    __syncthreads();
-    s = (sh[0] + sh[1]) + (sh[2] + sh[3]);
-    __syncthreads();
-
-    const bf16_t *row = logits + static_cast<int64_t>(b) * row_stride;
-    const bool vec_ok = ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
-    const float t_in = temperatures[b];
-    const bool greedy = (t_in == 0.f);
-    const float temp = greedy ? 1.f : t_in;
-    const int col0 = chunk * kSampChunk + threadIdx.x * 8;
-    float x[8];
-    load_x8(row, col0, vocab, temp, vec_ok, x);
-
-    float e[8];
-    if (greedy) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) e[i] = 1.f;
-    } else {
-        const float *nrow = noise + static_cast<int64_t>(b) * noise_row_stride;
-        if (((reinterpret_cast<uintptr_t>(nrow) & 15u) == 0) && col0 + 8 <= vocab) {
-            const float4 a = *reinterpret_cast<const float4 *>(nrow + col0);
-            const float4 c = *reinterpret_cast<const float4 *>(nrow + col0 + 4);
-            e[0] = a.x; e[1] = a.y; e[2] = a.z; e[3] = a.w;
-            e[4] = c.x; e[5] = c.y; e[6] = c.z; e[7] = c.w;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) e[i] = (col0 + i < vocab) ? nrow[col0 + i] : 1.f;
-        }
-    }
-
-    float best = -INFINITY;
-    int best_i = 0x7fffffff;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        if (col0 + i < vocab) {
-            float score;
-            if (greedy) {
-                score = x[i];
-            } else {
-                const float p = expf(x[i] - m) / s;
-                score = p / fmaxf(e[i], 1e-10f);
-            }
-            better(best, best_i, score, col0 + i);
-        }
-    }
-    // wavefront, then workgroup arg-max
+__device__ __forceinline__ void wave_best(float &best, int &best_i) {
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
         const float os = __shfl_xor(best, off, 64);
         const int oi = __shfl_xor(best_i, off, 64);
         better(best, best_i, os, oi);
     }
-    if (lane == 0) { sh[wave] = best; shi[wave] = best_i; }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; ++w) better(best, best_i, sh[w], shi[w]);
-        part_best[static_cast<int64_t>(b) * nchunks + chunk] = best;
-        part_idx[static_cast<int64_t>(b) * nchunks + chunk] = best_i;
+}
+
+// First index i in [0, 4) with w[i] > 0 whose running sum exceeds u * total; the last index of
+// positive weight when rounding leaves the target beyond the last running sum; -1 if no weight is
+// positive.  The same rule, level by level, is what the oracle restates in float64.
+__device__ __forceinline__ int pick4(const float (&w)[4], double u) {
+    const float total = (w[0] + w[1]) + (w[2] + w[3]);
+    const double t = u * static_cast<double>(total);
+    float run = 0.f;
+    int pick = -1, live = -1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        run += w[i];
+        if (w[i] > 0.f) {
+            live = i;
+            if (pick < 0 && static_cast<double>(run) > t) pick = i;
+        }
     }
+    return pick >= 0 ? pick : live;
 }
 
-// ---- in-kernel randomness: one uniform per row, inverse-CDF draw -----------------------------
-// Without a noise tensor to replay against, the exponential race is replaced by the textbook
-// draw from the same categorical distribution: with w_i = exp2((x_i - M) * log2(e)/T) and one
-// uniform u per row, the token is the first i (in column order) whose running sum of w exceeds
-// u * sum(w).  One Philox call per ROW instead of one random number and two logarithms per
-// column leaves a multiply, an exponential and an add per column -- the pass over the logits
-// runs at memory speed.
-//   pass A  per (8192-column chunk, row): chunk max m_c, s_c = sum exp2(y - m_c), and the chunk's
-//           arg-max (used by temperature-0 rows)                                -> workspace
-//   pass B  per row: M = max m_c, chunk weights s_c * exp2(m_c - M), their running sum picks
-//           the chunk; its 8192 logits are read once more (32 consecutive columns per lane), a
-//           workgroup scan picks the lane and the lane walks its columns        -> int64 token
-// Rounding can leave the target a hair beyond the last running sum; it then falls on the last
-// column of positive weight.  A row without any finite logit yields token 0.
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-constexpr int kCdfVec = 4;                                    // 16-byte loads per lane in pass A
-constexpr int kCdfChunk = kSampChunk * kCdfVec;               // 8192 columns per workgroup
-
-__host__ __device__ inline int cdf_chunks(int vocab) { return (vocab + kCdfChunk - 1) / kCdfChunk; }
-
-__device__ __forceinline__ float block_max4(float v, float *sh, int lane, int wave) {
-    v = wave_max(v);
-    __syncthreads();
-    if (lane == 0) sh[wave] = v;
-    __syncthreads();
-    return fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
-}
-
-__device__ __forceinline__ float block_sum4(float v, float *sh, int lane, int wave) {
-    v = wave_sum(v);
-    __syncthreads();
-    if (lane == 0) sh[wave] = v;
-    __syncthreads();
-    return (sh[0] + sh[1]) + (sh[2] + sh[3]);
-}
-
-__global__ __launch_bounds__(kSampThreads) void sampler_cdf_sums_kernel(
+template <bool kNoise>
+__global__ __launch_bounds__(kSampThreads) void sampler_chunk_kernel(
     const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
-    float *__restrict__ part_max, float *__restrict__ part_sum, float *__restrict__ part_best,
-    int32_t *__restrict__ part_idx, int32_t vocab, int32_t nchunks) {
+    const float *__restrict__ noise, int64_t noise_row_stride, uint64_t seed, uint64_t offset,
+    SampRecord *__restrict__ records, int32_t vocab, int32_t nchunks) {
     const int chunk = blockIdx.x;
     const int b = blockIdx.y;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
     const bf16_t *row = logits + static_cast<int64_t>(b) * row_stride;
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
     const float t_in = temperatures[b];
     const bool greedy = (t_in == 0.f);
-    const float k = greedy ? 1.f : 1.4426950408889634f / t_in;
-    u32x4_t raw[kCdfVec];
-    int col0[kCdfVec];
+
+    // ---- every load of the chunk goes out before the first use ----------------------------------
+    u32x4_t raw[kSampVec];
+    int col0[kSampVec];
+    bool full[kSampVec];
 #pragma unroll
-    for (int v = 0; v < kCdfVec; ++v) {
-        col0[v] = chunk * kCdfChunk + v * kSampChunk + threadIdx.x * 8;
+    for (int v = 0; v < kSampVec; ++v) {
+        col0[v] = chunk * kSampChunk + v * kSampSlice + tid * 8;
+        full[v] = vec_ok && col0[v] + 8 <= vocab;
         raw[v] = u32x4_t{0u, 0u, 0u, 0u};
-        // (streamed once: non-temporal, so that the rows do not displace one another in L2)
-        if (vec_ok && col0[v] + 8 <= vocab) raw[v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row + col0[v]));
+        if (full[v]) raw[v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row + col0[v]));
     }
-    float y[kCdfVec][8];
-    float m = -INFINITY;
+    float e[kSampVec][8];                                  // noise, where it is read
+    if (kNoise && !greedy) {
+        const float *nrow = noise + static_cast<int64_t>(b) * noise_row_stride;
+        const bool nvec_ok = ((reinterpret_cast<uintptr_t>(nrow) & 15u) == 0);
 #pragma unroll
-    for (int v = 0; v < kCdfVec; ++v) {
-        if (vec_ok && col0[v] + 8 <= vocab) {
-            unpack8(make_uint4(raw[v][0], raw[v][1], raw[v][2], raw[v][3]), y[v]);
+        for (int v = 0; v < kSampVec; ++v) {
+            if (nvec_ok && col0[v] + 8 <= vocab) {
+                const f32x4_t a = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(nrow + col0[v]));
+                const f32x4_t c = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(nrow + col0[v] + 4));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { e[v][i] = a[i]; e[v][4 + i] = c[i]; }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) e[v][i] = (col0[v] + i < vocab) ? nrow[col0[v] + i] : 1.f;
+            }
+        }
+    }
+    float x[kSampVec][8];                                  // columns past the row end read as -inf
+#pragma unroll
+    for (int v = 0; v < kSampVec; ++v) {
+        if (full[v]) {
+            unpack8(make_uint4(raw[v][0], raw[v][1], raw[v][2], raw[v][3]), x[v]);
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) y[v][i] = (col0[v] + i < vocab) ? bf16_to_f32(row[col0[v] + i]) : -INFINITY;
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            y[v][i] *= k;
-            m = fmaxf(m, y[v][i]);
+            for (int i = 0; i < 8; ++i) x[v][i] = (col0[v] + i < vocab) ? bf16_to_f32(row[col0[v] + i]) : -INFINITY;
         }
     }
-    __shared__ float sh[4];
-    __shared__ int shi[4];
-    if (greedy) {                                        // row-uniform branch: chunk arg-max, lowest column on ties
+
+    __shared__ float sh_max[kSampWaves];
+    __shared__ float sh_sum[kSampWaves][kSampVec];
+    __shared__ float sh_best[kSampWaves];
+    __shared__ int sh_col[kSampWaves];
+    SampRecord *rec = records + static_cast<int64_t>(b) * nchunks + chunk;
+
+    if (greedy) {                                          // row-uniform branch: chunk arg-max of the logits
         float best = -INFINITY;
-        int best_i = 0x7fffffff;
+        int best_i = kNoToken;
 #pragma unroll
-        for (int v = 0; v < kCdfVec; ++v)
+        for (int v = 0; v < kSampVec; ++v)
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                if (col0[v] + i < vocab && y[v][i] > best) { best = y[v][i]; best_i = col0[v] + i; }
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const float os = __shfl_xor(best, off, 64);
-            const int oi = __shfl_xor(best_i, off, 64);
-            better(best, best_i, os, oi);
-        }
-        if (lane == 0) { sh[wave] = best; shi[wave] = best_i; }
+                if (col0[v] + i < vocab && x[v][i] > best) { best = x[v][i]; best_i = col0[v] + i; }
+        wave_best(best, best_i);
+        if (lane == 0) { sh_best[wave] = best; sh_col[wave] = best_i; }
         __syncthreads();
-        if (threadIdx.x == 0) {
-            for (int w = 1; w < 4; ++w) better(best, best_i, sh[w], shi[w]);
-            part_best[static_cast<int64_t>(b) * nchunks + chunk] = best;
-            part_idx[static_cast<int64_t>(b) * nchunks + chunk] = best_i;
+        if (tid == 0) {
+            for (int w = 1; w < kSampWaves; ++w) better(best, best_i, sh_best[w], sh_col[w]);
+            *rec = SampRecord{0.f, 0.f, best, best_i};
         }
         return;
     }
-    m = block_max4(m, sh, lane, wave);
-    const float mm = (m == -INFINITY) ? 0.f : m;           // a chunk of -inf logits sums to 0
-    float ssum = 0.f;
-#pragma unroll
-    for (int v = 0; v < kCdfVec; ++v) {
-        float part = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) part += __builtin_amdgcn_exp2f(y[v][i] - mm);     // exp2(-inf) = 0 past the row end
-        ssum += part;
-    }
-    ssum = block_sum4(ssum, sh, lane, wave);
-    if (threadIdx.x == 0) {
-        part_max[static_cast<int64_t>(b) * nchunks + chunk] = m;
-        part_sum[static_cast<int64_t>(b) * nchunks + chunk] = ssum;
-    }
-}
 
-__global__ __launch_bounds__(kSampThreads) void sampler_cdf_select_kernel(
-    const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
-    uint64_t seed, uint64_t offset, const float *__restrict__ part_max, const float *__restrict__ part_sum,
-    const float *__restrict__ part_best, const int32_t *__restrict__ part_idx,
-    int64_t *__restrict__ out_tokens, int32_t vocab, int32_t nchunks) {
-    const int b = blockIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const float t_in = temperatures[b];
-    __shared__ float sh[4];
-    __shared__ int sh_pick[1];
-    if (t_in == 0.f) {                                   // greedy: best chunk, lowest column on ties
-        if (wave == 0) {
-            float best = -INFINITY;
-            int best_i = 0x7fffffff;
-            for (int c = lane; c < nchunks; c += kWave)
-                better(best, best_i, part_best[static_cast<int64_t>(b) * nchunks + c],
-                       part_idx[static_cast<int64_t>(b) * nchunks + c]);
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const float os = __shfl_xor(best, off, 64);
-                const int oi = __shfl_xor(best_i, off, 64);
-                better(best, best_i, os, oi);
-            }
-            if (lane == 0) out_tokens[b] = (best_i == 0x7fffffff) ? 0 : static_cast<int64_t>(best_i);
-        }
-        return;
-    }
+    // ---- x / T (noise: the reference's division; otherwise folded into the base-2 exponent) ------
     const float k = 1.4426950408889634f / t_in;
-    // ---- wavefront 0: row maximum, chunk weights relative to it, and the chunk that holds u * total ----
-    if (wave == 0) {
-        const float *pm = part_max + static_cast<int64_t>(b) * nchunks;
-        const float *ps = part_sum + static_cast<int64_t>(b) * nchunks;
-        float m = -INFINITY;
-        for (int c = lane; c < nchunks; c += kWave) m = fmaxf(m, pm[c]);
-        m = wave_max(m);
-        int pick = -2;                                   // -2: no finite logit in the row
-        float rest_in_chunk = 0.f;
-        if (m != -INFINITY) {
-            float total = 0.f;
-            for (int c = lane; c < nchunks; c += kWave) total += ps[c] * __builtin_amdgcn_exp2f(pm[c] - m);
-            total = wave_sum(total);
-            // one uniform per row, in (0, 1): 24 random bits plus one half
-            const uint2 key = make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
-            const uint4 r = Philox::draw(make_uint4(static_cast<uint32_t>(b), 0x5a17u, static_cast<uint32_t>(offset),
-                                                    static_cast<uint32_t>(offset >> 32)), key);
-            const float u = (static_cast<float>(r.x >> 8) + 0.5f) * 5.9604644775390625e-8f;
-            const float target = u * total;
-            // running sum in chunk order, 64 chunks at a time
-            float carry = 0.f;
-            int last_live = 0;
-            pick = -1;
-            for (int base = 0; base < nchunks; base += kWave) {
-                const int c = base + lane;
-                const float w = c < nchunks ? ps[c] * __builtin_amdgcn_exp2f(pm[c] - m) : 0.f;
-                float incl = w;
+    float m = -INFINITY;
 #pragma unroll
-                for (int off = 1; off < 64; off <<= 1) {
-                    const float up = __shfl_up(incl, off, 64);
-                    if (lane >= off) incl += up;
-                }
-                incl += carry;
-                const uint64_t live = __builtin_amdgcn_ballot_w64(w > 0.f);
-                const uint64_t hit = __builtin_amdgcn_ballot_w64(w > 0.f && incl > target);
-                if (live != 0) last_live = base + 63 - __builtin_clzll(live);
-                if (pick < 0 && hit != 0) {
-                    const int l = __builtin_ctzll(hit);
-                    pick = base + l;
-                    rest_in_chunk = target - __shfl(incl - w, l, 64);     // what is left to walk inside the chunk
-                }
-                carry = __shfl(incl, 63, 64);
-            }
-            if (pick < 0) { pick = last_live; rest_in_chunk = INFINITY; }   // rounding: beyond the last running sum
-        }
-        if (lane == 0) { sh_pick[0] = pick; sh[0] = rest_in_chunk; sh[1] = m; }
-    }
-    __syncthreads();
-    const int chunk = sh_pick[0];
-    const float rest = sh[0];
-    const float m = sh[1];
-    if (chunk == -2) {
-        if (threadIdx.x == 0) out_tokens[b] = 0;
-        return;
-    }
-    // ---- inside the chunk: 32 consecutive columns per lane, scan over the 256 lanes -------------
-    const bf16_t *row = logits + static_cast<int64_t>(b) * row_stride;
-    const int c0 = chunk * kCdfChunk + threadIdx.x * 32;
-    float w[32];
-    float mine = 0.f;
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        float x[8];
-        const int cc = c0 + v * 8;
-        if (((reinterpret_cast<uintptr_t>(row + cc) & 15u) == 0) && cc + 8 <= vocab) {
-            unpack8(*reinterpret_cast<const uint4 *>(row + cc), x);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) x[i] = (cc + i < vocab) ? bf16_to_f32(row[cc + i]) : -INFINITY;
-        }
+    for (int v = 0; v < kSampVec; ++v)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            w[v * 8 + i] = __builtin_amdgcn_exp2f(x[i] * k - m);
-            mine += w[v * 8 + i];
+            x[v][i] = kNoise ? x[v][i] / t_in : x[v][i] * k;
+            m = fmaxf(m, x[v][i]);
         }
+    m = wave_max(m);
+    if (lane == 0) sh_max[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(sh_max[0], sh_max[1]), fmaxf(sh_max[2], sh_max[3]));
+    const float mm = (m == -INFINITY) ? 0.f : m;           // a chunk of -inf logits: every weight is 0
+
+    if (kNoise) {
+        float ssum = 0.f, best = -INFINITY;
+        int best_i = kNoToken;
+#pragma unroll
+        for (int v = 0; v < kSampVec; ++v)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float ex = expf(x[v][i] - mm);       // exp(-inf) = 0 past the row end
+                ssum += ex;
+                if (col0[v] + i < vocab) better(best, best_i, ex / fmaxf(e[v][i], 1e-10f), col0[v] + i);
+            }
+        ssum = wave_sum(ssum);
+        wave_best(best, best_i);
+        if (lane == 0) { sh_sum[wave][0] = ssum; sh_best[wave] = best; sh_col[wave] = best_i; }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < kSampWaves; ++w) better(best, best_i, sh_best[w], sh_col[w]);
+            *rec = SampRecord{m, (sh_sum[0][0] + sh_sum[1][0]) + (sh_sum[2][0] + sh_sum[3][0]), best, best_i};
+        }
+        return;
     }
-    // inclusive scan of `mine` over the workgroup, in lane order
-    float incl = mine;
+
+    // ---- no noise tensor: weights, and the draw inside the chunk -----------------------------------
+    // (the counter is wave-uniform, so the generator runs on the scalar unit beside the exponentials)
+    const uint4 r = Philox::draw(make_uint4(static_cast<uint32_t>(b), 0x10000u + static_cast<uint32_t>(chunk),
+                                            static_cast<uint32_t>(offset), static_cast<uint32_t>(offset >> 32)),
+                                 make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)));
+    float part[kSampVec];                                  // this lane's 8-column sums, one per slice
+#pragma unroll
+    for (int v = 0; v < kSampVec; ++v) {
+        float p = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            x[v][i] = __builtin_amdgcn_exp2f(x[v][i] - mm);    // from here on x holds the weights
+            p += x[v][i];
+        }
+        part[v] = p;
+    }
+#pragma unroll
+    for (int v = 0; v < kSampVec; ++v) {
+        const float ws = wave_sum(part[v]);
+        if (lane == 0) sh_sum[wave][v] = ws;
+    }
+    __syncthreads();
+    float slice_sum[kSampVec];
+#pragma unroll
+    for (int v = 0; v < kSampVec; ++v) slice_sum[v] = (sh_sum[0][v] + sh_sum[1][v]) + (sh_sum[2][v] + sh_sum[3][v]);
+    const float chunk_sum = (slice_sum[0] + slice_sum[1]) + (slice_sum[2] + slice_sum[3]);
+    const int vsel = pick4(slice_sum, unit_uniform(r.x));                     // workgroup-uniform
+    if (vsel < 0) {                                        // no positive weight: the chunk can never be chosen
+        if (tid == 0) *rec = SampRecord{m, 0.f, 0.f, min(chunk * kSampChunk, vocab - 1)};
+        return;
+    }
+    const float wsum[kSampWaves] = {sh_sum[0][vsel], sh_sum[1][vsel], sh_sum[2][vsel], sh_sum[3][vsel]};
+    const int wsel = pick4(wsum, unit_uniform(r.y));                          // > = 0: the slice has weight
+    if (wave != wsel) return;                              // (wave-uniform; no barrier follows)
+    const float mine = vsel == 0 ? part[0] : vsel == 1 ? part[1] : vsel == 2 ? part[2] : part[3];
+    float incl = mine;                                     // inclusive scan over the 64 lanes
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
         const float up = __shfl_up(incl, off, 64);
         if (lane >= off) incl += up;
     }
-    if (lane == 63) sh[wave] = incl;
-    __syncthreads();
-    for (int wv = 0; wv < wave; ++wv) incl += sh[wv];
-    // owner: the first lane whose running sum exceeds `rest` (its span then contains it); if rounding
-    // put `rest` beyond the chunk's total, the last lane of positive weight
-    int first = (mine > 0.f && incl > rest) ? static_cast<int>(threadIdx.x) : 0x7fffffff;
-    int live = (mine > 0.f) ? static_cast<int>(threadIdx.x) : -1;
+    const double t3 = unit_uniform(r.z) * static_cast<double>(__shfl(incl, 63, 64));
+    const uint64_t live = __builtin_amdgcn_ballot_w64(mine > 0.f);            // != 0: the wavefront has weight
+    const uint64_t hit = __builtin_amdgcn_ballot_w64(mine > 0.f && static_cast<double>(incl) > t3);
+    const int lsel = hit != 0 ? __builtin_ctzll(hit) : 63 - __builtin_clzll(live);
+    if (lane != lsel) return;
+    float w8[8];
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        first = min(first, __shfl_xor(first, off, 64));
-        live = max(live, __shfl_xor(live, off, 64));
-    }
-    __shared__ int sh_first[4], sh_live[4];
-    if (lane == 0) { sh_first[wave] = first; sh_live[wave] = live; }
-    __syncthreads();
-    first = min(min(sh_first[0], sh_first[1]), min(sh_first[2], sh_first[3]));
-    live = max(max(sh_live[0], sh_live[1]), max(sh_live[2], sh_live[3]));
-    const int owner = first != 0x7fffffff ? first : live;
-    if (owner < 0) {                                     // every weight of the chunk underflowed: its first column
-        if (threadIdx.x == 0) out_tokens[b] = min(chunk * kCdfChunk, vocab - 1);
-        return;
-    }
-    if (static_cast<int>(threadIdx.x) == owner) {
-        float run = incl - mine;
-        int tok = -1, last = c0;
+    for (int i = 0; i < 8; ++i)
+        w8[i] = vsel == 0 ? x[0][i] : vsel == 1 ? x[1][i] : vsel == 2 ? x[2][i] : x[3][i];
+    float total = 0.f;
 #pragma unroll
-        for (int j = 0; j < 32; ++j) {
-            if (w[j] > 0.f) last = c0 + j;
-            if (tok < 0 && w[j] > 0.f && run + w[j] > rest) tok = c0 + j;
-            run += w[j];
+    for (int i = 0; i < 8; ++i) total += w8[i];
+    const double t4 = unit_uniform(r.w) * static_cast<double>(total);
+    float run = 0.f;
+    int isel = -1, ilive = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        run += w8[i];
+        if (w8[i] > 0.f) {
+            ilive = i;
+            if (isel < 0 && static_cast<double>(run) > t4) isel = i;
         }
-        out_tokens[b] = tok < 0 ? last : tok;
     }
+    if (isel < 0) isel = ilive;
+    *rec = SampRecord{m, chunk_sum, 0.f, chunk * kSampChunk + vsel * kSampSlice + tid * 8 + isel};
 }
 
-__global__ __launch_bounds__(kWave) void sampler_pick_kernel(
-    const float *__restrict__ part_best, const int32_t *__restrict__ part_idx,
-    int64_t *__restrict__ out_tokens, int32_t nchunks) {
-    const int b = blockIdx.x;
-    float best = -INFINITY;
-    int best_i = 0x7fffffff;
-    for (int c = threadIdx.x; c < nchunks; c += kWave)
-        better(best, best_i, part_best[static_cast<int64_t>(b) * nchunks + c],
-               part_idx[static_cast<int64_t>(b) * nchunks + c]);
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float os = __shfl_xor(best, off, 64);
-        const int oi = __shfl_xor(best_i, off, 64);
-        better(best, best_i, os, oi);
+// One wavefront per row: merges the row's chunk records into the token.
+__global__ __launch_bounds__(kSampThreads) void sampler_row_kernel(
+    const SampRecord *__restrict__ records, const float *__restrict__ temperatures, int32_t with_noise,
+    uint64_t seed, uint64_t offset, int64_t *__restrict__ out_tokens, int32_t batch, int32_t nchunks) {
+    const int lane = threadIdx.x & 63;
+    const int b = blockIdx.x * kSampWaves + (threadIdx.x >> 6);
+    if (b >= batch) return;                                // wave-uniform; the kernel has no barrier
+    const SampRecord *rec = records + static_cast<int64_t>(b) * nchunks;
+    const float t_in = temperatures[b];
+    if (t_in == 0.f || with_noise) {
+        // greedy: best logit; noise: best of exp(x - m_c) / E scaled to the row maximum and row sum
+        float m = -INFINITY;
+        if (t_in != 0.f) {
+            for (int c = lane; c < nchunks; c += kWave) m = fmaxf(m, rec[c].m);
+            m = wave_max(m);
+        }
+        float s = 0.f;
+        if (t_in != 0.f && m != -INFINITY) {
+            for (int c = lane; c < nchunks; c += kWave) s += rec[c].s * expf(rec[c].m - m);
+            s = wave_sum(s);
+        }
+        float best = -INFINITY;
+        int best_i = kNoToken;
+        for (int c = lane; c < nchunks; c += kWave) {
+            const SampRecord r = rec[c];
+            if (r.col == kNoToken) continue;
+            float score = r.best;
+            if (t_in != 0.f) score = (m == -INFINITY) ? 0.f : r.best * expf(r.m - m) / s;
+            better(best, best_i, score, r.col);
+        }
+        wave_best(best, best_i);
+        if (lane == 0) out_tokens[b] = (best_i == kNoToken) ? 0 : static_cast<int64_t>(best_i);
+        return;
     }
-    if (threadIdx.x == 0) out_tokens[b] = (best_i == 0x7fffffff) ? 0 : static_cast<int64_t>(best_i);
+    // ---- no noise tensor: the chunk is drawn by the chunk weights, the column inside it is in the record
+    float m = -INFINITY;
+    for (int c = lane; c < nchunks; c += kWave) m = fmaxf(m, rec[c].m);
+    m = wave_max(m);
+    if (m == -INFINITY) {                                  // no finite logit in the row
+        if (lane == 0) out_tokens[b] = 0;
+        return;
+    }
+    double total = 0.0;
+    for (int c = lane; c < nchunks; c += kWave)
+        total += static_cast<double>(rec[c].s * __builtin_amdgcn_exp2f(rec[c].m - m));
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) total += __shfl_xor(total, off, 64);
+    const uint4 r = Philox::draw(make_uint4(static_cast<uint32_t>(b), 0x5a17u, static_cast<uint32_t>(offset),
+                                            static_cast<uint32_t>(offset >> 32)),
+                                 make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)));
+    const double target = unit_uniform(r.x) * total;
+    double carry = 0.0;
+    int pick = -1, last_live = -1;
+    for (int base = 0; base < nchunks; base += kWave) {    // running sum in chunk order, 64 chunks at a time
+        const int c = base + lane;
+        const float w = c < nchunks ? rec[c].s * __builtin_amdgcn_exp2f(rec[c].m - m) : 0.f;
+        double incl = static_cast<double>(w);
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const double up = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += up;
+        }
+        incl += carry;
+        const uint64_t live = __builtin_amdgcn_ballot_w64(w > 0.f);
+        const uint64_t hit = __builtin_amdgcn_ballot_w64(w > 0.f && incl > target);
+        if (live != 0) last_live = base + 63 - __builtin_clzll(live);
+        if (pick < 0 && hit != 0) pick = base + __builtin_ctzll(hit);
+        carry = __shfl(incl, 63, 64);
+    }
+    if (pick < 0) pick = last_live;                        // rounding: the target lies beyond the last running sum
+    if (lane == 0) out_tokens[b] = pick < 0 ? 0 : static_cast<int64_t>(rec[pick].col);
+}
+
+static int launch_sample(const bf16_t *logits, int64_t logits_row_stride, const float *temperatures,
+                         const float *noise, int64_t noise_row_stride, uint64_t seed, uint64_t offset,
+                         int64_t *out_tokens, SampRecord *records, int32_t batch, int32_t vocab, hipStream_t s) {
+    const int nchunks = samp_chunks(vocab);
+    if (noise)
+        hipLaunchKernelGGL(sampler_chunk_kernel<true>, dim3(nchunks, batch), dim3(kSampThreads), 0, s, logits,
+                           logits_row_stride, temperatures, noise, noise_row_stride, seed, offset, records, vocab, nchunks);
+    else
+        hipLaunchKernelGGL(sampler_chunk_kernel<false>, dim3(nchunks, batch), dim3(kSampThreads), 0, s, logits,
+                           logits_row_stride, temperatures, noise, noise_row_stride, seed, offset, records, vocab, nchunks);
+    if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
+    hipLaunchKernelGGL(sampler_row_kernel, dim3((batch + kSampWaves - 1) / kSampWaves), dim3(kSampThreads), 0, s, records,
+                       temperatures, noise ? 1 : 0, seed, offset, out_tokens, batch, nchunks);
+    return launch_status();
+}
+
+static int check_sample_args(const void *logits, int64_t logits_row_stride, const float *temperatures,
+                             const float *noise, int64_t noise_row_stride, const int64_t *out_tokens,
+                             int32_t batch, int32_t vocab) {
+    if (batch < 0 || vocab <= 0) return NVA_ERR_BAD_SHAPE;
+    if (batch > 65535) return NVA_ERR_BAD_SHAPE;
+    if (batch == 0) return NVA_OK;
+    if (!logits || !temperatures || !out_tokens) return NVA_ERR_NULL_POINTER;
+    if (logits_row_stride < vocab) return NVA_ERR_BAD_STRIDE;
+    if (noise && noise_row_stride < vocab) return NVA_ERR_BAD_STRIDE;
+    return NVA_OK;
 }
 
 }  // namespace nva
 
 extern "C" size_t nva_sample_workspace_bytes(int32_t batch, int32_t vocab) {
     if (batch <= 0 || vocab <= 0) return 0;
-    return static_cast<size_t>(batch) * nva::samp_chunks(vocab) * 4 * sizeof(float);
+    return static_cast<size_t>(batch) * nva::samp_chunks(vocab) * sizeof(nva::SampRecord);
 }
 
 extern "C" int nva_sample(const void *logits, int64_t logits_row_stride, const float *temperatures,
@@ -483,40 +409,13 @@ extern "C" int nva_sample(const void *logits, int64_t logits_row_stride, const f
                           int64_t *out_tokens, void *workspace, size_t workspace_bytes, int32_t batch,
                           int32_t vocab, void *stream) {
     using namespace nva;
-    if (batch < 0 || vocab <= 0) return NVA_ERR_BAD_SHAPE;
-    if (batch == 0) return NVA_OK;
-    if (batch > 65535) return NVA_ERR_BAD_SHAPE;
-    if (!logits || !temperatures || !out_tokens || !workspace) return NVA_ERR_NULL_POINTER;
-    if (logits_row_stride < vocab) return NVA_ERR_BAD_STRIDE;
-    if (noise && noise_row_stride < vocab) return NVA_ERR_BAD_STRIDE;
+    const int rc = check_sample_args(logits, logits_row_stride, temperatures, noise, noise_row_stride, out_tokens,
+                                     batch, vocab);
+    if (rc != NVA_OK || batch == 0) return rc;
+    if (!workspace) return NVA_ERR_NULL_POINTER;
     if (!aligned16(workspace)) return NVA_ERR_MISALIGNED;
     if (workspace_bytes < nva_sample_workspace_bytes(batch, vocab)) return NVA_ERR_WORKSPACE_TOO_SMALL;
-    const int nchunks = samp_chunks(vocab);
-    const size_t n = static_cast<size_t>(batch) * nchunks;
-    float *part_max = static_cast<float *>(workspace);
-    float *part_sum = part_max + n;
-    float *part_best = part_sum + n;
-    int32_t *part_idx = reinterpret_cast<int32_t *>(part_best + n);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const bf16_t *lg = static_cast<const bf16_t *>(logits);
-    if (noise == nullptr) {
-        const int cchunks = cdf_chunks(vocab);                 // fewer, wider chunks: fits the same workspace
-        hipLaunchKernelGGL(sampler_cdf_sums_kernel, dim3(cchunks, batch), dim3(kSampThreads), 0, s, lg,
-                           logits_row_stride, temperatures, part_max, part_sum, part_best, part_idx, vocab, cchunks);
-        if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
-        hipLaunchKernelGGL(sampler_cdf_select_kernel, dim3(batch), dim3(kSampThreads), 0, s, lg, logits_row_stride,
-                           temperatures, seed, offset, part_max, part_sum, part_best, part_idx, out_tokens, vocab,
-                           cchunks);
-        return launch_status();
-    }
-    hipLaunchKernelGGL(sampler_partials_kernel, dim3(nchunks, batch), dim3(kSampThreads), 0, s, lg,
-                       logits_row_stride, temperatures, part_max, part_sum, vocab, nchunks);
-    if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL(sampler_argmax_kernel, dim3(nchunks, batch), dim3(kSampThreads), 0, s, lg,
-                       logits_row_stride, temperatures, noise, noise_row_stride, part_max,
-                       part_sum, part_best, part_idx, vocab, nchunks);
-    if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL(sampler_pick_kernel, dim3(batch), dim3(kWave), 0, s, part_best, part_idx, out_tokens,
-                       nchunks);
-    return launch_status();
+    return launch_sample(static_cast<const bf16_t *>(logits), logits_row_stride, temperatures, noise, noise_row_stride,
+                         seed, offset, out_tokens, static_cast<SampRecord *>(workspace), batch, vocab,
+                         static_cast<hipStream_t>(stream));
 }

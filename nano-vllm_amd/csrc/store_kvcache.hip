@@ -4,32 +4,47 @@
 // i (D = num_kv_heads*head_dim bf16 elements of K and of V) is copied bit-exactly to row
 // slot_mapping[i] of the flat caches; slot -1 skips the row.
 //
-// Layout / mapping: one workgroup of 256 lanes per token.  A row is D*2/16 16-byte chunks
-// (128 for D = 1024); lanes 0..127 copy the K chunks and lanes 128..255 the V chunks, so each
-// (token, head) row of 256 B is written by 16 consecutive lanes, one dwordx4 store per lane.  The kernel
-// is pure HBM traffic: D*2 B read + D*2 B written per tensor per stored token.
+// Layout / mapping: a row is D*2/16 16-byte chunks (128 for D = 1024); a workgroup of 256 lanes
+// takes kScatterTokens consecutive tokens, lanes [0, chunks) moving the K chunks and lanes
+// [chunks, 2*chunks) the V chunks of each, so every (token, head) row of 256 B is written by 16
+// consecutive lanes with one dwordx4 store per lane.  The kernel is pure HBM traffic (D*2 B read +
+// D*2 B written per tensor per stored token) and, at 4096 tokens, short enough that latency
+// decides: the row loads do not depend on the slot ids, so all of a lane's loads -- the slot ids
+// and kScatterTokens row chunks -- are issued together and only the stores wait for the slots
+// (rows whose slot turns out to be -1 are read in vain).  The cache rows are not read again by
+// this kernel: non-temporal stores.
 #include "nva_common.h"
 
 namespace nva {
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kScatterTokens = 4;      // tokens per workgroup = independent 16-byte loads in flight per lane
+
 __global__ __launch_bounds__(256) void store_kvcache_kernel(
-    const uint4 *__restrict__ key, int64_t key_stride16,      // row strides in 16-byte units
-    const uint4 *__restrict__ value, int64_t value_stride16,
-    uint4 *__restrict__ k_cache, uint4 *__restrict__ v_cache,
-    const int32_t *__restrict__ slot_mapping, int32_t chunks_per_row, int64_t num_slots) {
-    const int64_t token = blockIdx.x;
-    const int64_t slot = slot_mapping[token];
-    if (slot < 0 || slot >= num_slots) return;   // -1 = skip (attention.py:22); never write OOB
-    const uint4 *ksrc = key + token * key_stride16;
-    const uint4 *vsrc = value + token * value_stride16;
-    uint4 *kdst = k_cache + slot * chunks_per_row;
-    uint4 *vdst = v_cache + slot * chunks_per_row;
+    const u32x4_t *__restrict__ key, int64_t key_stride16,      // row strides in 16-byte units
+    const u32x4_t *__restrict__ value, int64_t value_stride16,
+    u32x4_t *__restrict__ k_cache, u32x4_t *__restrict__ v_cache,
+    const int32_t *__restrict__ slot_mapping, int32_t n_tokens, int32_t chunks_per_row, int64_t num_slots) {
+    const int64_t token0 = static_cast<int64_t>(blockIdx.x) * kScatterTokens;
     // lanes [0, chunks) move K, lanes [chunks, 2*chunks) move V: wave-uniform for D = 1024
     for (int c = threadIdx.x; c < 2 * chunks_per_row; c += blockDim.x) {
         const bool is_v = c >= chunks_per_row;
         const int cc = is_v ? c - chunks_per_row : c;
-        const uint4 row = is_v ? vsrc[cc] : ksrc[cc];
-        (is_v ? vdst : kdst)[cc] = row;
+        const u32x4_t *src = is_v ? value : key;
+        const int64_t stride = is_v ? value_stride16 : key_stride16;
+        u32x4_t *dst = is_v ? v_cache : k_cache;
+        int64_t slot[kScatterTokens];
+        u32x4_t row[kScatterTokens];
+#pragma unroll
+        for (int t = 0; t < kScatterTokens; ++t) {
+            const int64_t token = token0 + t < n_tokens ? token0 + t : n_tokens - 1;   // past the end: re-read the last row
+            slot[t] = token0 + t < n_tokens ? slot_mapping[token] : -1;
+            row[t] = __builtin_nontemporal_load(src + token * stride + cc);
+        }
+#pragma unroll
+        for (int t = 0; t < kScatterTokens; ++t)      // -1 = skip (attention.py:22); never write out of bounds
+            if (slot[t] >= 0 && slot[t] < num_slots) __builtin_nontemporal_store(row[t], dst + slot[t] * chunks_per_row + cc);
     }
 }
 
@@ -51,11 +66,12 @@ extern "C" int nva_store_kvcache(const void *key, int64_t key_row_stride,
         !nva::aligned16(v_cache))
         return NVA_ERR_MISALIGNED;
     const int32_t chunks = static_cast<int32_t>(d / 8);
-    hipLaunchKernelGGL(nva::store_kvcache_kernel, dim3(n_tokens), dim3(256), 0,
+    const int32_t groups = (n_tokens + nva::kScatterTokens - 1) / nva::kScatterTokens;
+    hipLaunchKernelGGL(nva::store_kvcache_kernel, dim3(groups), dim3(256), 0,
                        static_cast<hipStream_t>(stream),
-                       static_cast<const uint4 *>(key), key_row_stride / 8,
-                       static_cast<const uint4 *>(value), value_row_stride / 8,
-                       static_cast<uint4 *>(k_cache), static_cast<uint4 *>(v_cache),
-                       slot_mapping, chunks, num_slots);
+                       static_cast<const nva::u32x4_t *>(key), key_row_stride / 8,
+                       static_cast<const nva::u32x4_t *>(value), value_row_stride / 8,
+                       static_cast<nva::u32x4_t *>(k_cache), static_cast<nva::u32x4_t *>(v_cache),
+                       slot_mapping, n_tokens, chunks, num_slots);
     return nva::launch_status();
 }

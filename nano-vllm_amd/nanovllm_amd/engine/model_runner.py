@@ -241,6 +241,7 @@ class ModelRunner:
         _lib.check(rc, "nva_stage_decode_inputs")
         for graph in self.graphs[bucket]:                         # later segments are enqueued while the first runs
             graph.replay()
+        reset_context()                                           # a decode step: the head must not gather by a prefill step's cu_seqlens_q
         return self.model.compute_logits(self.graph_vars["outputs"][:bs])
 
     def can_launch_ahead(self, num_seqs: int) -> bool:

@@ -1,8 +1,11 @@
 """Token sampler backed by the fused gfx950 kernels.
 
-Drop-in for nanovllm/layers/sampler.py: ``Sampler()(logits, temperatures) -> int64 [B]``,
-an exact categorical draw from ``softmax(logits / T)`` via the exponential race
-``argmax(p / E)``, ``E ~ Exp(1)``.
+Drop-in for nanovllm/layers/sampler.py: ``Sampler()(logits, temperatures) -> int64 [B]``, a
+categorical draw from ``softmax(logits / T)``.  Given a tensor of ``E ~ Exp(1)`` draws the kernels
+evaluate the reference's exponential race ``argmax(p / E)`` (replayable); without one -- what the
+module interface does -- they draw from the same distribution by a tree of inverse-CDF steps with
+Philox uniforms of 32 bits per level (conditional probabilities below 2**-32 are not resolved;
+the reference's fp32 race has a comparable floor).
 """
 from __future__ import annotations
 
@@ -19,8 +22,8 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor, noise: Optional[tor
     """``argmax(softmax(logits.float() / T) / clamp_min(E, 1e-10))`` per row.
 
     ``noise`` (fp32 ``[B, V]``) supplies ``E`` explicitly so a draw can be replayed; with
-    ``noise=None`` the kernel draws the token from the same categorical distribution by inverse
-    CDF with one Philox uniform per row keyed by ``(seed, offset)``.
+    ``noise=None`` the kernel draws the token from the same categorical distribution by a tree of
+    inverse-CDF steps (chunk, slice, group, column) with Philox uniforms keyed by ``(seed, offset)``.
     Rows with temperature 0 return ``argmax(logits)``.
     """
     assert logits.dim() == 2 and logits.dtype == torch.bfloat16 and logits.stride(1) == 1

@@ -14,9 +14,11 @@ here: GQA mapping ``h_kv = h_q // (Hq // Hkv)``, paged layout ``[num_blocks, pag
 bottom-right aligned causal mask when ``seqlen_k > seqlen_q`` (flash-attn >= 2.1), fp32
 softmax/accumulation and zero output for rows that see no keys.
 
-For draws without a noise tensor the library's own scheme is restated as well: one Philox4x32-10
-uniform per row (``philox4x32_10``, ``row_uniforms``; pinned by the Random123 known-answer vectors)
-walked through float64 running sums of the softmax (``inverse_cdf_bounds``).
+For draws without a noise tensor the library's own scheme is restated as well: a tree of
+inverse-CDF draws over the columns (``tree_draw``: row -> chunk -> slice -> group -> 8 columns ->
+column), every level with its own Philox4x32-10 uniform (``philox4x32_10``, ``row_uniforms``; pinned
+by the Random123 known-answer vectors), each level a walk through float64 running sums
+(``inverse_cdf_bounds`` is the one-level form).
 
 Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
 import this package, and only as the checker / the timed CPU baseline.  Nothing under the
@@ -35,6 +37,7 @@ from .hotpath import (  # noqa: F401
     philox4x32_10,
     row_uniforms,
     inverse_cdf_bounds,
+    tree_draw,
     sample,
     sample_scores,
 )

@@ -146,7 +146,7 @@ def baseline(cfg, prompts: List[List[int]], params, num_requests: int = 16, max_
                 break
     dt = time.perf_counter() - t0
     return {"value": round(done / dt, 2), "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"first {num_requests} requests of the bench mix, outputs capped at {max_new_tokens} tokens "
-                      f"({done} of {total} output tokens generated in {dt:.1f} s); same scheduler and block "
+            "sample": f"{num_requests} requests ({done} of {total} output tokens generated in {dt:.1f} s, "
+                      f"{sum(len(p) for p in prompts[:num_requests])} prompt tokens); same scheduler and block "
                       "manager, eager torch CPU ops (bf16 SDPA attention, index_copy scatter, eager sampler)",
             "seconds": round(dt, 2)}

@@ -209,16 +209,24 @@ def philox4x32_10(counter, key):
     return c
 
 
+def _unit_uniform(word):
+    """32 random bits -> uniform in (0, 1): ``(word + 1/2) * 2**-32`` (exact in float64)."""
+    return (int(word) + 0.5) * 2.0 ** -32
+
+
+def _philox_words(seed, offset, row, stream):
+    return philox4x32_10((row, stream, offset & 0xFFFFFFFF, (offset >> 32) & 0xFFFFFFFF),
+                         (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))
+
+
 def row_uniforms(seed, offset, batch):
-    """The uniform in (0, 1) that the library draws for row ``b`` of a call keyed by
-    ``(seed, offset)`` when no noise tensor is given: first output word of Philox4x32-10 with
-    counter ``(b, 0x5a17, offset_lo, offset_hi)`` and key ``(seed_lo, seed_hi)``; its top 24 bits
-    plus one half, times 2**-24.  float64 ``[batch]``."""
+    """The uniform in (0, 1) that the library draws at the ROW level (which 8192-column chunk) for
+    row ``b`` of a call keyed by ``(seed, offset)`` when no noise tensor is given: first output word
+    of Philox4x32-10 with counter ``(b, 0x5a17, offset_lo, offset_hi)`` and key
+    ``(seed_lo, seed_hi)``, plus one half, times 2**-32.  float64 ``[batch]``."""
     out = torch.empty(batch, dtype=torch.float64)
     for b in range(batch):
-        r = philox4x32_10((b, 0x5A17, offset & 0xFFFFFFFF, (offset >> 32) & 0xFFFFFFFF),
-                          (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))
-        out[b] = ((r[0] >> 8) + 0.5) * 2.0 ** -24
+        out[b] = _unit_uniform(_philox_words(seed, offset, b, 0x5A17)[0])
     return out
 
 
@@ -228,3 +236,64 @@ def inverse_cdf_bounds(logits, temperatures):
     categorical distribution as the exponential race of nanovllm/layers/sampler.py:12-14."""
     p = torch.softmax(logits.double() / temperatures.double().unsqueeze(1), dim=-1)
     return p.cumsum(-1)
+
+
+# The library's draw without a noise tensor is a tree of such inverse-CDF draws over the columns in
+# column order, each level with its own uniform: row -> chunk of 8192 columns -> slice of 2048 ->
+# group of 512 -> group of 8 -> column.
+TREE_CHUNK = 8192
+TREE_FANOUT = (4, 4, 64, 8)          # slices per chunk, groups per slice, 8-column groups per group, columns
+
+
+def _pick(weights, u):
+    """Inverse-CDF step over a float64 weight vector: first index of positive weight whose running
+    sum exceeds ``u * total`` (the last index of positive weight if rounding leaves none).  Also
+    returns how far ``u`` lies from the nearer edge of the chosen interval, as a probability."""
+    total = float(weights.sum())
+    live = (weights > 0).nonzero().flatten()
+    if live.numel() == 0:
+        return -1, float("inf")
+    incl = weights.cumsum(0)
+    t = u * total
+    hit = ((weights > 0) & (incl > t)).nonzero().flatten()
+    idx = int(hit[0]) if hit.numel() else int(live[-1])
+    hi = float(incl[idx]) / total
+    lo = hi - float(weights[idx]) / total
+    return idx, min(abs(u - lo), abs(hi - u))
+
+
+def tree_draw(logits, temperatures, seed, offset):
+    """float64 restatement of the library's draw from ``softmax(logits / T)`` without a noise
+    tensor -- the same distribution as nanovllm/layers/sampler.py:12-14, by other randomness.
+
+    Row ``b`` picks a chunk of 8192 columns by the chunk weights with ``row_uniforms``; inside chunk
+    ``c`` the four output words of Philox counter ``(b, 0x10000 + c, offset)`` pick, in turn, one of
+    4 slices of 2048 columns, one of 4 groups of 512, one of 64 groups of 8 and one of 8 columns,
+    each by its share of the level's weight.  Returns ``(tokens int64 [B], margins float64 [B])``:
+    the margin is the smallest distance, over the levels, between a level's uniform and the edges
+    of the interval it fell into -- where it is tiny, fp32 sums may legitimately pick the neighbour.
+    A row without a finite logit yields token 0.
+    """
+    batch, vocab = logits.shape
+    nchunks = -(-vocab // TREE_CHUNK)
+    tokens = torch.zeros(batch, dtype=torch.int64)
+    margins = torch.full((batch,), float("inf"), dtype=torch.float64)
+    for b in range(batch):
+        y = logits[b].double() / float(temperatures[b])
+        top = float(y.max())
+        if top == float("-inf"):
+            continue
+        w = torch.zeros(nchunks * TREE_CHUNK, dtype=torch.float64)
+        w[:vocab] = torch.exp(y - top)
+        c, margin = _pick(w.view(nchunks, -1).sum(-1), _unit_uniform(_philox_words(seed, offset, b, 0x5A17)[0]))
+        words = _philox_words(seed, offset, b, 0x10000 + c)
+        node, col = w[c * TREE_CHUNK:(c + 1) * TREE_CHUNK], c * TREE_CHUNK
+        for fan, word in zip(TREE_FANOUT, words):
+            node = node.view(fan, -1)
+            i, mg = _pick(node.sum(-1), _unit_uniform(word))
+            margin = min(margin, mg)
+            col += i * node.shape[1]
+            node = node[i]
+        tokens[b] = col
+        margins[b] = margin
+    return tokens, margins

@@ -129,7 +129,7 @@ def test_prefill_validation():
 def test_sampler_validation_and_workspace_size():
     lib = _lib.load()
     ws = lib.nva_sample_workspace_bytes
-    assert ws(256, 151936) == 256 * 75 * 16 and ws(1, 1) == 16 and ws(0, 10) == 0
+    assert ws(256, 151936) == 256 * 19 * 16 and ws(1, 1) == 16 and ws(2, 8193) == 64 and ws(0, 10) == 0   # one 16-byte record per 8192-column chunk
     f = lib.nva_sample
     assert f(None, 100, A, None, 0, 0, 0, A, A, 1 << 20, 4, 100, None) == _lib.ERR_NULL_POINTER
     assert f(A, 100, A, None, 0, 0, 0, A, None, 1 << 20, 4, 100, None) == _lib.ERR_NULL_POINTER

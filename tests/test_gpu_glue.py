@@ -102,6 +102,49 @@ def test_qk_norm_rope_fused_scatter_matches_store_kvcache(dev):
     assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2) and bool(kc1.any()) and bool(vc1.any())
 
 
+@pytest.mark.parametrize("hq,hkv", [(16, 8), (32, 8)])
+def test_fused_scatter_is_bit_exact_against_the_oracle_scatter(dev, hq, hkv):
+    """The scatter the engine really runs -- nva_qk_norm_rope with cache pointers -- on the slot
+    mapping of the scatter benchmark configuration (4096 tokens into 512 blocks x 256 slots, 5 %
+    skipped, value rows strided inside the fused qkv buffer), against oracle.store_kvcache:
+      * V cache bit-exact (the rows are copied unchanged);
+      * K cache bit-exact against the oracle scatter of the key rows the kernel returned (slot
+        indexing), and those rows against the oracle's norm + rope to the glue tolerance (most bits equal);
+      * every slot that was not addressed is still zero."""
+    import oracle
+    from nanovllm_amd import synthetic
+    case = synthetic.scatter_case(seed=0)
+    n, d = case.slot_mapping.numel(), 128
+    g = torch.Generator().manual_seed(77)
+    qkv = torch.randn(n, (hq + 2 * hkv) * d, generator=g).to(torch.bfloat16)
+    qw = (1 + 0.2 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    kw = (1 + 0.2 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    pos = torch.randint(0, 4096, (n,), generator=g)
+    rope = glue.build_rope_cache(d, 4096, 1e6)
+    slots = case.slot_mapping
+    kc = torch.zeros(512, 256, hkv, d, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    q, k, v = layers.qk_norm_rope(qkv.to(dev), pos.to(dev), qw.to(dev), kw.to(dev), rope.to(dev), hq, hkv, d, 1e-6,
+                                  kv_store=(kc, vc, slots.to(dev)))
+    torch.cuda.synchronize()
+    wq, wk, wv = glue.qk_norm_rope(qkv, pos, qw, kw, rope, hq, hkv, d, 1e-6)
+    ek, ev = torch.zeros(512, 256, hkv, d, dtype=torch.bfloat16), torch.zeros(512, 256, hkv, d, dtype=torch.bfloat16)
+    oracle.store_kvcache(wk.contiguous(), wv, ek, ev, slots)
+    as_bits = lambda t: t.cpu().contiguous().view(torch.int16)
+    assert torch.equal(as_bits(vc), as_bits(ev))                                  # values: bit-exact
+    ek2, ev2 = torch.zeros_like(ek), torch.zeros_like(ev)
+    oracle.store_kvcache(k.cpu(), v.cpu(), ek2, ev2, slots)
+    assert torch.equal(as_bits(kc), as_bits(ek2)) and torch.equal(as_bits(vc), as_bits(ev2))   # slot indexing: bit-exact
+    same = float((as_bits(kc) == as_bits(ek)).float().mean())
+    assert same >= 0.97, same                                                      # keys: the oracle's bits almost everywhere
+    diff = (kc.cpu().float() - ek.float()).abs()
+    assert float(diff.max()) <= 2.0 ** -6 * float(ek.float().abs().max())
+    untouched = torch.ones(512 * 256, dtype=torch.bool)
+    untouched[slots[slots >= 0].long()] = False
+    assert not bool(kc.cpu().view(512 * 256, -1)[untouched].any()) and not bool(vc.cpu().view(512 * 256, -1)[untouched].any())
+    assert int((slots >= 0).sum()) == case.n_valid
+
+
 @pytest.mark.gpu
 def test_stage_decode_inputs_copies_and_hands_over_tokens(dev):
     """The staging kernel copies the pinned buffer bit for bit and replaces exactly the input

@@ -341,3 +341,44 @@ def test_inverse_cdf_draws_the_softmax():
     freq = torch.bincount(tok, minlength=row.shape[1]).double() / n
     p = torch.softmax(row[0].double() / 0.7, -1)
     assert float((freq - p).abs().max()) <= 1.0 / n + 1e-12
+
+
+def test_tree_draw_reduces_to_one_inverse_cdf_on_eight_columns():
+    """With at most 8 columns only the last level of the tree has a choice, so the draw must be the
+    plain inverse CDF of that level's uniform: word 3 of Philox counter (row, 0x10000, offset)."""
+    g = torch.Generator().manual_seed(8)
+    batch, seed, offset = 300, 0xABCDEF0123, 41
+    logits = (torch.randn(batch, 8, generator=g) * 1.5).to(torch.bfloat16)
+    logits[::7, 2] = float("-inf")
+    temps = torch.linspace(0.4, 1.6, batch)
+    tok, margin = oracle.tree_draw(logits, temps, seed, offset)
+    bounds = oracle.inverse_cdf_bounds(logits, temps)
+    u = torch.tensor([(oracle.philox4x32_10((b, 0x10000, offset, 0), (seed & 0xFFFFFFFF, seed >> 32))[3] + 0.5) * 2.0 ** -32
+                      for b in range(batch)], dtype=torch.float64)
+    want = torch.searchsorted(bounds, u.unsqueeze(1), right=True).squeeze(1)
+    sure = margin > 1e-9
+    assert int(sure.sum()) >= batch - 2 and torch.equal(tok[sure], want[sure])
+    assert bool((logits[torch.arange(batch), tok] > float("-inf")).all())
+
+
+def test_tree_draw_is_categorical_across_all_levels():
+    """Heavy columns placed so that every level of the tree has to choose (different chunks, slices,
+    groups of 512, groups of 8 and neighbours inside a group of 8): empirical frequencies over many
+    rows against softmax(logits / T), chi-square."""
+    cols = [3, 5, 6, 11, 700, 2050, 2051, 4100, 8191, 8192, 9000, 16390, 19999]
+    vocab, n, t = 20000, 12000, 0.9
+    row = torch.full((vocab,), float("-inf"))
+    vals = torch.tensor([1.0, 0.5, 2.0, 0.0, 1.5, -0.5, 0.25, 1.0, 0.75, 2.0, -1.0, 1.25, 0.5])
+    row[cols] = vals
+    logits = row.to(torch.bfloat16).expand(n, vocab)
+    tok, _ = oracle.tree_draw(logits, torch.full((n,), t), seed=99, offset=5)
+    p = torch.softmax(vals.double() / t, -1)
+    index = {c: i for i, c in enumerate(cols)}
+    assert all(int(x) in index for x in tok.tolist())            # never a column of zero weight
+    freq = torch.bincount(torch.tensor([index[int(x)] for x in tok.tolist()]), minlength=len(cols)).double()
+    chi2 = float(((freq - n * p) ** 2 / (n * p)).sum())
+    assert chi2 < 45.0, chi2                                      # 12 dof: P(chi2 > 45) ~ 1e-5
+    # a different offset is a different draw; the same key reproduces it
+    again, _ = oracle.tree_draw(logits[:50], torch.full((50,), t), seed=99, offset=5)
+    other, _ = oracle.tree_draw(logits[:50], torch.full((50,), t), seed=99, offset=6)
+    assert torch.equal(again, tok[:50]) and not torch.equal(other, tok[:50])
