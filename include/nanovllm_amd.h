@@ -33,7 +33,8 @@ enum nva_status {
     NVA_ERR_MISALIGNED = 5,           /* base pointer not 16-byte aligned                   */
     NVA_ERR_WORKSPACE_TOO_SMALL = 6,  /* workspace_bytes below *_workspace_bytes()          */
     NVA_ERR_LAUNCH_FAILED = 7,        /* hipGetLastError() after the launch was not success */
-    NVA_ERR_NO_DEVICE = 8             /* no HIP device visible                              */
+    NVA_ERR_NO_DEVICE = 8,            /* no HIP device visible                              */
+    NVA_ERR_SCRATCH_TOO_SMALL = 9     /* problem exceeds the library's built-in scratch array */
 };
 
 /* Library version, (major << 16) | minor. */
@@ -177,6 +178,27 @@ int nva_sample(const void *logits, int64_t logits_row_stride,
                int64_t *out_tokens,
                void *workspace, size_t workspace_bytes,
                int32_t batch, int32_t vocab, void *stream);
+
+/*
+ * nva_sample without a workspace argument, for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, kernels and results as nva_sample; the per-chunk
+ * records live in a device array built into the library (2 MiB per GPU the library is used on, held
+ * until the process ends), which bounds the problem size:
+ *     batch * ceil(vocab / 8192) <= NVA_SAMPLE_STATIC_MAX_RECORDS      (6898 rows at vocab 151,936)
+ * Larger problems return NVA_ERR_SCRATCH_TOO_SMALL and launch nothing.  The call allocates and frees
+ * nothing; the first call on a device looks the array's address up (make that call outside stream
+ * capture).  All calls on one GPU share the array: calls that overlap in time on one GPU race and
+ * must be ordered by the caller (one stream, or events); nothing needs clearing between calls.
+ */
+#define NVA_SAMPLE_STATIC_MAX_RECORDS 131072
+
+int nva_sample_static(const void *logits, int64_t logits_row_stride,
+                      const float *temperatures,
+                      const float *noise, int64_t noise_row_stride,
+                      uint64_t seed, uint64_t offset,
+                      int64_t *out_tokens,
+                      int32_t batch, int32_t vocab, void *stream);
 
 /*
  * ---- steps either side of the hot path (the callers' element-wise glue) ----------------

@@ -14,6 +14,7 @@ extern "C" const char *nva_status_string(int status) {
         case NVA_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
         case NVA_ERR_LAUNCH_FAILED: return "kernel launch failed";
         case NVA_ERR_NO_DEVICE: return "no HIP device";
+        case NVA_ERR_SCRATCH_TOO_SMALL: return "problem exceeds the built-in scratch array";
         default: return "unknown status";
     }
 }

@@ -38,6 +38,8 @@
 
 #include <math.h>
 
+#include <mutex>
+
 namespace nva {
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -418,4 +420,58 @@ extern "C" int nva_sample(const void *logits, int64_t logits_row_stride, const f
     return launch_sample(static_cast<const bf16_t *>(logits), logits_row_stride, temperatures, noise, noise_row_stride,
                          seed, offset, out_tokens, static_cast<SampRecord *>(workspace), batch, vocab,
                          static_cast<hipStream_t>(stream));
+}
+
+// ---- the same sampler for callers that cannot allocate --------------------------------------------
+// The chunk records live in a file-scope device array instead of a caller-supplied workspace.  Each
+// GPU the library runs on holds its own copy of the array (2 MiB) until the process ends.  In host
+// code the array's name is only a handle: its device address is looked up once per device with
+// hipGetSymbolAddress and that pointer is what the kernels receive.
+namespace nva {
+
+constexpr int kStaticRecords = NVA_SAMPLE_STATIC_MAX_RECORDS;
+constexpr int kMaxDevices = 64;
+
+static __device__ __align__(256) unsigned char scratch[static_cast<size_t>(kStaticRecords) * sizeof(SampRecord)];
+
+static std::mutex g_scratch_mutex;
+static SampRecord *g_scratch_ptr[kMaxDevices] = {};       // device address of `scratch` on each device
+
+// Device address of this device's copy of `scratch`; nullptr (and *status set) on failure.
+static SampRecord *static_scratch(int *status) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        *status = NVA_ERR_NO_DEVICE;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+            (void)hipGetLastError();
+            *status = NVA_ERR_LAUNCH_FAILED;
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = static_cast<SampRecord *>(ptr);
+    }
+    return g_scratch_ptr[dev];
+}
+
+}  // namespace nva
+
+extern "C" int nva_sample_static(const void *logits, int64_t logits_row_stride, const float *temperatures,
+                                 const float *noise, int64_t noise_row_stride, uint64_t seed, uint64_t offset,
+                                 int64_t *out_tokens, int32_t batch, int32_t vocab, void *stream) {
+    using namespace nva;
+    const int rc = check_sample_args(logits, logits_row_stride, temperatures, noise, noise_row_stride, out_tokens,
+                                     batch, vocab);
+    if (rc != NVA_OK || batch == 0) return rc;
+    if (static_cast<int64_t>(batch) * samp_chunks(vocab) > kStaticRecords) return NVA_ERR_SCRATCH_TOO_SMALL;
+    int status = NVA_OK;
+    SampRecord *records = static_scratch(&status);
+    if (records == nullptr) return status;
+    // every record the row kernel reads is written by the chunk kernel of the same call: nothing to clear
+    return launch_sample(static_cast<const bf16_t *>(logits), logits_row_stride, temperatures, noise, noise_row_stride,
+                         seed, offset, out_tokens, records, batch, vocab, static_cast<hipStream_t>(stream));
 }

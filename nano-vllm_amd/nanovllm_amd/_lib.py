@@ -21,6 +21,7 @@ ERR_MISALIGNED = 5
 ERR_WORKSPACE_TOO_SMALL = 6
 ERR_LAUNCH_FAILED = 7
 ERR_NO_DEVICE = 8
+ERR_SCRATCH_TOO_SMALL = 9
 
 _vp, _i32, _i64, _u64, _f32, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_uint64, C.c_float, C.c_size_t
 
@@ -45,6 +46,7 @@ SIGNATURES = {
     "nva_silu_and_mul": (C.c_int, [_vp, _i64, _vp, _i32, _i32, _vp]),
     "nva_stage_decode_inputs": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _i32, _vp, _i32, _vp]),
     "nva_sample": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _u64, _u64, _vp, _vp, _sz, _i32, _i32, _vp]),
+    "nva_sample_static": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _u64, _u64, _vp, _i32, _i32, _vp]),
 }
 
 _lib = None

@@ -32,8 +32,8 @@ def test_library_exports_every_declared_symbol():
 def test_version_and_status_strings():
     lib = _lib.load()
     assert lib.nva_version() >= 1
-    seen = {_lib.status_string(c) for c in range(9)}
-    assert len(seen) == 9 and _lib.status_string(0) == "ok"
+    seen = {_lib.status_string(c) for c in range(10)}
+    assert len(seen) == 10 and _lib.status_string(0) == "ok"
     assert _lib.status_string(1234) == "unknown status"
 
 
@@ -175,3 +175,16 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libnanovllm_amd.so")
     with pytest.raises(_lib.HipLibraryMissing, match="no CPU fallback"):
         _lib.load()
+
+
+def test_sample_static_validation():
+    """The allocation-free sampler rejects bad arguments and problems beyond its built-in scratch
+    array before it touches a device."""
+    f = _lib.load().nva_sample_static
+    # (logits, row_stride, temperatures, noise, noise_stride, seed, offset, out_tokens, batch, vocab, stream)
+    assert f(None, 100, A, None, 0, 0, 0, A, 4, 100, None) == _lib.ERR_NULL_POINTER
+    assert f(A, 99, A, None, 0, 0, 0, A, 4, 100, None) == _lib.ERR_BAD_STRIDE
+    assert f(A, 100, A, None, 0, 0, 0, A, 4, 0, None) == _lib.ERR_BAD_SHAPE
+    assert f(A, 100, A, None, 0, 0, 0, A, 0, 100, None) == _lib.OK
+    assert f(A, 151936, A, None, 0, 0, 0, A, 6899, 151936, None) == _lib.ERR_SCRATCH_TOO_SMALL    # 6899 * 19 records > 131072
+    assert f(A, 1 << 30, A, None, 0, 0, 0, A, 2, 1 << 30, None) == _lib.ERR_SCRATCH_TOO_SMALL     # 2 * 131072 records
