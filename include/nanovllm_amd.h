@@ -158,11 +158,11 @@ int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride,
  * temperatures: fp32 [batch].  T == 0 selects greedy argmax(logits) for that row (an
  * extension; the reference forbids T <= 1e-10, nanovllm/sampling_params.py:11).
  * noise: fp32 [batch, vocab] Exp(1) draws (row stride noise_row_stride): the formula above is
- * evaluated (scores relative to the maximum of each 8192-column chunk, rescaled to the row) and a
+ * evaluated (scores relative to the maximum of each 2048-column chunk, rescaled to the row) and a
  * draw can be replayed; the argmax differs from the formula only between scores that agree to fp32
  * rounding.  NULL: the token is drawn from the same categorical distribution softmax(logits / T) by a
- * tree of inverse-CDF steps over the columns in column order (row -> chunk of 8192 -> slice of 2048
- * -> group of 512 -> group of 8 -> column; at every level the first branch whose running sum of
+ * tree of inverse-CDF steps (row -> chunk of 8192 columns -> one of 4 column groups -> one of its 64
+ * lanes -> one of the lane's 32 columns; at every level the first branch whose running sum of
  * weights exceeds u * total), each level with its own 32-bit uniform from Philox4x32-10 keyed by
  * (seed, offset, row, chunk); the same (seed, offset) reproduces the draw.  Sums are fp32 and a
  * conditional probability below 2^-32 at a level is not resolved.
@@ -185,7 +185,7 @@ int nva_sample(const void *logits, int64_t logits_row_stride,
  * counterpart in the reference.  Same arguments, kernels and results as nva_sample; the per-chunk
  * records live in a device array built into the library (2 MiB per GPU the library is used on, held
  * until the process ends), which bounds the problem size:
- *     batch * ceil(vocab / 8192) <= NVA_SAMPLE_STATIC_MAX_RECORDS      (6898 rows at vocab 151,936)
+ *     batch * ceil(vocab / 2048) <= NVA_SAMPLE_STATIC_MAX_RECORDS      (1747 rows at vocab 151,936)
  * Larger problems return NVA_ERR_SCRATCH_TOO_SMALL and launch nothing.  The call allocates and frees
  * nothing; the first call on a device looks the array's address up (make that call outside stream
  * capture).  All calls on one GPU share the array: calls that overlap in time on one GPU race and

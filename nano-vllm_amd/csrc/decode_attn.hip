@@ -41,7 +41,7 @@
 //
 // HBM traffic per sequence and layer: ctx * num_kv_heads * 128 * 2 B for K plus the same for
 // V (4096 B per token at 8 kv heads).  Partials: at most (W + batch*num_kv_heads) * G rows of 520 B;
-// the stored split: 64 KB of worker records and 8 bytes per sequence.
+// the stored split: 64 KB of worker records, 8 bytes per sequence and 8 bytes per (sequence, kv head) pair.
 #include "nva_common.h"
 
 #include <math.h>
@@ -82,6 +82,7 @@ struct DecodeArgs {
     int32_t *pref_out;       // [batch + 1] stage-count prefix sums, written for the merge kernel
     int32_t *ctx_out;        // [batch] clipped context lengths       } the work split, kept for later
     int32_t *rec_out;        // [kDecWorkers][8] first stage per worker } launches over the same contexts
+    int32_t *pair_out;       // [batch * num_kv_heads][2] first partial row and number of partials of every pair
     float *part_ml;          // [rows][2]
     float *part_o;           // [rows][128]
     int32_t batch, max_blocks, num_heads, num_kv_heads, num_blocks;
@@ -413,40 +414,69 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
 
 // Merges the partials of every (sequence, kv head) pair that was split over several workers.
 // One workgroup of G wavefronts per pair: wavefront h merges query head g*G + h, lane = 2 dims.
-// It recomputes which workers met the pair from the stage-count prefix sums the streaming
-// kernel left in the workspace; pairs seen by a single worker were already written.
-template <int G>
+// Which workers met the pair follows from the stage-count prefix sums the streaming kernel left in
+// the workspace; pairs seen by a single worker were already written.  The building call also leaves
+// (first partial row, number of partials) per pair in the workspace, so that a call that reuses the
+// work split starts from one 8-byte read instead of three dependent ones.  The partials of a pair
+// are fetched eight at a time, all loads of a round in flight together.
+template <int G, bool kReuse>
 __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArgs a) {
     const int pair = blockIdx.x;
     const int b = pair / a.num_kv_heads;
     const int g = pair % a.num_kv_heads;
     const int h = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
-    const int64_t n_total = a.pref_out[a.batch];
-    const int pb = a.pref_out[b];
-    const int nst = (a.pref_out[b + 1] - pb) / a.num_kv_heads;
-    if (nst == 0) return;                              // no keys: the zero rows are already there
-    const int64_t n_workers = n_total < kDecWorkers ? n_total : kDecWorkers;
-    const int64_t pair_lo = pb + static_cast<int64_t>(g) * nst;
-    const int w_first = worker_of(pair_lo, n_total, n_workers);
-    const int n_parts = worker_of(pair_lo + nst - 1, n_total, n_workers) - w_first + 1;
-    if (n_parts == 1) return;                          // one worker saw the whole pair and wrote it
-    const int64_t row0 = (static_cast<int64_t>(w_first) + pair) * G + h;   // rows of consecutive workers are G apart
-    float mx = -INFINITY;
-    for (int pi = lane; pi < n_parts; pi += kWave) mx = fmaxf(mx, a.part_ml[(row0 + static_cast<int64_t>(pi) * G) * 2]);
-    mx = wave_max(mx);
-    float acc0 = 0.f, acc1 = 0.f, lsum = 0.f;
-    if (mx > -INFINITY) {
-        // eight partials in flight per lane: a pair met by many workers (small batches) is otherwise one dependent
-        // memory round trip per partial (measured: 22 -> 18 us per call at batch 16; more unrolling is slower again)
-#pragma unroll 8
-        for (int pi = 0; pi < n_parts; ++pi) {
-            const int64_t at = row0 + static_cast<int64_t>(pi) * G;
-            const float f = exp2f(a.part_ml[at * 2] - mx);
-            lsum = fmaf(f, a.part_ml[at * 2 + 1], lsum);
-            const float2 o2 = *reinterpret_cast<const float2 *>(a.part_o + at * kHeadDim + 2 * lane);
-            acc0 = fmaf(f, o2.x, acc0);
-            acc1 = fmaf(f, o2.y, acc1);
+    int64_t row0;
+    int n_parts;
+    if constexpr (kReuse) {
+        const int2 info = reinterpret_cast<const int2 *>(a.pair_out)[pair];
+        row0 = static_cast<int64_t>(info.x) + h;
+        n_parts = info.y;
+    } else {
+        const int64_t n_total = a.pref_out[a.batch];
+        const int pb = a.pref_out[b];
+        const int nst = (a.pref_out[b + 1] - pb) / a.num_kv_heads;
+        n_parts = 0;                                   // no keys: the zero rows are already there
+        row0 = 0;
+        if (nst > 0) {
+            const int64_t n_workers = n_total < kDecWorkers ? n_total : kDecWorkers;
+            const int64_t pair_lo = pb + static_cast<int64_t>(g) * nst;
+            const int w_first = worker_of(pair_lo, n_total, n_workers);
+            n_parts = worker_of(pair_lo + nst - 1, n_total, n_workers) - w_first + 1;
+            row0 = (static_cast<int64_t>(w_first) + pair) * G;   // rows of consecutive workers are G apart
+        }
+        if (threadIdx.x == 0) reinterpret_cast<int2 *>(a.pair_out)[pair] = int2{static_cast<int>(row0), n_parts};
+        row0 += h;
+    }
+    if (n_parts <= 1) return;                          // one worker saw the whole pair and wrote it
+    float mx = -INFINITY, lsum = 0.f, acc0 = 0.f, acc1 = 0.f;
+    for (int base = 0; base < n_parts; base += 8) {
+        float pm[8], pl[8];
+        float2 po[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int64_t at = row0 + static_cast<int64_t>(min(base + j, n_parts - 1)) * G;
+            const float2 ml = *reinterpret_cast<const float2 *>(a.part_ml + at * 2);
+            po[j] = *reinterpret_cast<const float2 *>(a.part_o + at * kHeadDim + 2 * lane);
+            pm[j] = base + j < n_parts ? ml.x : -INFINITY;
+            pl[j] = ml.y;
+        }
+        float m_new = mx;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) m_new = fmaxf(m_new, pm[j]);
+        if (m_new > -INFINITY) {
+            const float keep = exp2f(mx - m_new);      // 0 in the first round
+            lsum *= keep;
+            acc0 *= keep;
+            acc1 *= keep;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float f = exp2f(pm[j] - m_new);  // 0 for slots past the last partial
+                lsum = fmaf(f, pl[j], lsum);
+                acc0 = fmaf(f, po[j].x, acc0);
+                acc1 = fmaf(f, po[j].y, acc1);
+            }
+            mx = m_new;
         }
     }
     const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
@@ -461,16 +491,19 @@ static int launch_decode(const DecodeArgs &a, bool reuse, hipStream_t stream) {
     else
         hipLaunchKernelGGL((decode_stream_kernel<G, false>), dim3(kDecGrid), dim3(kDecThreads), 0, stream, a);
     if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
-    hipLaunchKernelGGL(decode_merge_kernel<G>, dim3(a.batch * a.num_kv_heads), dim3(G * kWave), 0, stream, a);
+    if (reuse)
+        hipLaunchKernelGGL((decode_merge_kernel<G, true>), dim3(a.batch * a.num_kv_heads), dim3(G * kWave), 0, stream, a);
+    else
+        hipLaunchKernelGGL((decode_merge_kernel<G, false>), dim3(a.batch * a.num_kv_heads), dim3(G * kWave), 0, stream, a);
     return launch_status();
 }
 
 static inline size_t align_up(size_t v, size_t to) { return (v + to - 1) / to * to; }
 
 struct DecodeWorkspace {
-    size_t pref_bytes, ctx_bytes, rec_bytes, rows, total;
+    size_t pref_bytes, ctx_bytes, rec_bytes, pair_bytes, rows, total;
 };
-static DecodeWorkspace decode_workspace(int32_t batch, int32_t num_heads, int32_t head_dim) {
+static DecodeWorkspace decode_workspace(int32_t batch, int32_t num_heads, int32_t num_kv_heads, int32_t head_dim) {
     DecodeWorkspace ws;
     const size_t per_launch = static_cast<size_t>(batch < kDecMaxBatch ? batch : kDecMaxBatch);
     ws.pref_bytes = align_up((per_launch + 1) * sizeof(int32_t), 256);
@@ -479,7 +512,8 @@ static DecodeWorkspace decode_workspace(int32_t batch, int32_t num_heads, int32_
     ws.rows = static_cast<size_t>(kDecWorkers) * (num_heads < 8 ? num_heads : 8) + per_launch * num_heads;
     ws.ctx_bytes = align_up(per_launch * sizeof(int32_t), 256);
     ws.rec_bytes = static_cast<size_t>(kDecWorkers) * 8 * sizeof(int32_t);
-    ws.total = ws.pref_bytes + ws.ctx_bytes + ws.rec_bytes +
+    ws.pair_bytes = align_up(per_launch * static_cast<size_t>(num_kv_heads) * 2 * sizeof(int32_t), 256);
+    ws.total = ws.pref_bytes + ws.ctx_bytes + ws.rec_bytes + ws.pair_bytes +
                ws.rows * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
     return ws;
 }
@@ -490,7 +524,8 @@ extern "C" size_t nva_paged_decode_workspace_bytes(int32_t batch, int32_t num_he
                                                    int32_t max_blocks) {
     (void)max_blocks;
     if (batch <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
-    return nva::decode_workspace(batch, num_heads, head_dim).total;
+    // (the number of kv heads is not an argument: sized for the most there can be, one per query head)
+    return nva::decode_workspace(batch, num_heads, num_heads, head_dim).total;
 }
 
 extern "C" int nva_paged_decode_attn(const void *q, int64_t q_row_stride, const void *k_cache,
@@ -531,8 +566,8 @@ extern "C" int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride
     if (bt_row_stride < max_blocks) return NVA_ERR_BAD_STRIDE;
     if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(workspace) || !aligned16(out))
         return NVA_ERR_MISALIGNED;
-    const DecodeWorkspace ws = decode_workspace(batch, num_heads, head_dim);
-    if (workspace_bytes < ws.total) return NVA_ERR_WORKSPACE_TOO_SMALL;
+    if (workspace_bytes < nva_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks)) return NVA_ERR_WORKSPACE_TOO_SMALL;
+    const DecodeWorkspace ws = decode_workspace(batch, num_heads, num_kv_heads, head_dim);
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     DecodeArgs a;
@@ -543,7 +578,8 @@ extern "C" int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride
     a.pref_out = static_cast<int32_t *>(workspace);
     a.ctx_out = reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + ws.pref_bytes);
     a.rec_out = reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + ws.pref_bytes + ws.ctx_bytes);
-    a.part_ml = reinterpret_cast<float *>(static_cast<char *>(workspace) + ws.pref_bytes + ws.ctx_bytes + ws.rec_bytes);
+    a.pair_out = reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + ws.pref_bytes + ws.ctx_bytes + ws.rec_bytes);
+    a.part_ml = reinterpret_cast<float *>(static_cast<char *>(workspace) + ws.pref_bytes + ws.ctx_bytes + ws.rec_bytes + ws.pair_bytes);
     // every launch of a split batch overwrites the stored work split, so only a single launch can reuse it
     const bool reuse = plan == NVA_PLAN_REUSE && batch <= kDecMaxBatch;
     a.part_o = a.part_ml + ws.rows * 2;

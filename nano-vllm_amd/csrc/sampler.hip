@@ -4,35 +4,39 @@
 //     x = float(logits) / T;  p = softmax(x);  token = argmax_i p_i / max(E_i, 1e-10)
 //
 // A row of 151,936 logits is far too little work for one workgroup and 64..256 rows are too few
-// workgroups for 256 CUs, so a row is cut into chunks of 8192 columns (one workgroup of 256 lanes,
-// four 16-byte loads of 8 bf16 per lane, all issued before the first use, non-temporal: the logits
-// are read exactly once).  sampler_chunk_kernel leaves one 16-byte record per (row, chunk);
+// workgroups for 256 CUs, so a row is cut into chunks (one workgroup of 256 lanes each, 16-byte
+// loads of 8 bf16 per lane, all issued before the first use, non-temporal: the logits are read
+// exactly once).  sampler_chunk_kernel leaves one 16-byte record per (row, chunk);
 // sampler_row_kernel (one wavefront per row) merges a row's records into the token.
 //
-// With a caller-supplied tensor of E ~ Exp(1) draws (replayable; used for parity) the score of
-// column i is evaluated relative to the CHUNK maximum m_c, e_i = exp(x_i - m_c) / max(E_i, 1e-10)
-// with the reference's true fp32 division by T, and the record keeps (m_c, sum exp, best e_i, its
-// column).  The row merge scales every chunk's best by exp(m_c - M) / S: the same quantity
-// softmax(x)_i / E_i the reference maximises, factored as exp(x_i - m_c) * exp(m_c - M) instead of
-// exp(x_i - M), so the argmax can differ from the reference only where two scores agree to within
-// a few fp32 roundings.  Ties go to the lowest column, as torch.argmax does.
+// With a caller-supplied tensor of E ~ Exp(1) draws (replayable; used for parity; chunks of 2048
+// columns) the score of column i is evaluated relative to the CHUNK maximum m_c,
+// e_i = exp(x_i - m_c) / max(E_i, 1e-10) with the reference's true fp32 division by T, and the
+// record keeps (m_c, sum exp, best e_i, its column).  The row merge scales every chunk's best by
+// exp(m_c - M) / S: the same quantity softmax(x)_i / E_i the reference maximises, factored as
+// exp(x_i - m_c) * exp(m_c - M) instead of exp(x_i - M), so the argmax can differ from the
+// reference only where two scores agree to within a few fp32 roundings.  Ties go to the lowest
+// column, as torch.argmax does.
 //
-// Without a noise tensor (what serving uses) there is nothing to replay against, and the token is
-// drawn from the same categorical distribution softmax(x) by a tree of inverse-CDF draws over the
-// columns in column order, every level with a uniform of its own (32 random bits, compared in
-// double precision; a conditional probability below 2^-32 at some level is therefore not
-// resolved, and sums are fp32):
-//     row      -> chunk (8192 columns)   by the chunk weights s_c * exp2(m_c - M)   [row kernel]
-//     chunk    -> slice (2048 columns)   by the four slice sums                     [chunk kernel]
-//     slice    -> wavefront (512)        by the four wavefront sums
-//     wavefront-> lane (8 columns)       by an inclusive scan over the 64 lanes
-//     lane     -> column                 by a walk over its 8 weights
-// The four in-chunk levels run in the chunk kernel on the weights it already holds in registers,
-// so the logits are read once and the row kernel touches only the records.  Uniforms come from
-// Philox4x32-10 keyed by (seed, offset): counter (row, 0x5a17, offset) for the row level, counter
-// (row, 0x10000 + chunk, offset) for the four levels inside a chunk (one output word each).
-// Temperature 0 = greedy argmax of the logits (an extension; nanovllm/sampling_params.py:11
-// forbids it).  A row without any finite logit yields token 0.
+// Without a noise tensor (what serving uses; chunks of 8192 columns) there is nothing to replay
+// against, and the token is drawn from the same categorical distribution softmax(x) by a tree of
+// inverse-CDF draws, every level with a uniform of its own (32 random bits, compared in double
+// precision; a conditional probability below 2^-32 at some level is therefore not resolved, and
+// sums are fp32):
+//     row       -> chunk (8192 columns)  by the chunk weights s_c * exp2(m_c - M)   [row kernel]
+//     chunk     -> wavefront             by the four wavefront sums                 [chunk kernel]
+//     wavefront -> lane                  by an inclusive scan over the 64 lane sums
+//     lane      -> column                by a walk over the lane's 32 weights
+// (lane t of a chunk owns columns 2048 v + 8 t + [0, 8) for v = 0..3, walked in that order).  The
+// three in-chunk levels run in the chunk kernel, so the logits are read once and the row kernel
+// touches only the records.  Only the packed bf16 logits stay in registers across the workgroup
+// reductions (16 registers instead of 32 weights); for the last level the chosen lane hands them
+// to its wavefront through LDS and 32 lanes recompute one weight each, bit for bit as summed
+// (a serial walk by one lane costs a full wavefront's instruction stream, +40 % kernel time).
+// Uniforms come from Philox4x32-10 keyed by (seed, offset): counter (row, 0x5a17, offset) for the
+// row level, counter (row, 0x10000 + chunk, offset) for the levels inside a chunk (one output
+// word each).  Temperature 0 = greedy argmax of the logits (an extension;
+// nanovllm/sampling_params.py:11 forbids it).  A row without any finite logit yields token 0.
 // Algorithmic HBM bytes per row: vocab * 2 B (+ vocab * 4 B when the noise is read).
 #include "nva_common.h"
 
@@ -47,12 +51,12 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kSampThreads = 256;
 constexpr int kSampWaves = kSampThreads / kWave;
-constexpr int kSampVec = 4;                               // 16-byte logit loads per lane
-constexpr int kSampSlice = kSampThreads * 8;              // 2048 columns: one load of the whole workgroup
-constexpr int kSampChunk = kSampSlice * kSampVec;         // 8192 columns per workgroup
+constexpr int kSampSlice = kSampThreads * 8;              // 2048 columns: one 16-byte load per lane
+constexpr int kDrawVec = 4;                               // no noise tensor: four loads per lane, 8192 columns per workgroup
+constexpr int kNoiseVec = 1;                              // with noise: 2048 columns per workgroup (8 logits + 8 noise values per lane)
 constexpr int kNoToken = 0x7fffffff;
 
-__host__ __device__ inline int samp_chunks(int vocab) { return (vocab + kSampChunk - 1) / kSampChunk; }
+__host__ __device__ inline int samp_chunks(int vocab, int vec) { return (vocab + kSampSlice * vec - 1) / (kSampSlice * vec); }
 
 // One record per (row, chunk), written by the chunk kernel and read by the row kernel.
 //   noise:   {m_c, sum exp(x - m_c), best exp(x - m_c) / max(E, 1e-10), its column}
@@ -115,7 +119,29 @@ __device__ __forceinline__ int pick4(const float (&w)[4], double u) {
     return pick >= 0 ? pick : live;
 }
 
-template <bool kNoise>
+// Makes the compiler forget what it knows about the packed logits, so that code after this point
+// unpacks them again instead of keeping the 32 floats of an earlier pass alive in registers.
+template <int kVec>
+__device__ __forceinline__ void forget(u32x4_t (&raw)[kVec]) {
+#pragma unroll
+    for (int v = 0; v < kVec; ++v) asm volatile("" : "+v"(raw[v]));
+}
+
+// The 8 packed bf16 logits of columns [col0, col0 + 8): one 16-byte non-temporal load where the
+// row allows it, else element by element; columns past the row end read as -inf (bf16 0xFF80).
+__device__ __forceinline__ u32x4_t load_columns8(const bf16_t *row, bool vec_ok, int col0, int vocab) {
+    if (vec_ok && col0 + 8 <= vocab) return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row + col0));
+    uint32_t h[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = (col0 + i < vocab) ? row[col0 + i] : 0xFF80u;
+    return u32x4_t{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+}
+
+__device__ __forceinline__ void columns8(const u32x4_t &raw, float (&x)[8]) {
+    unpack8(make_uint4(raw[0], raw[1], raw[2], raw[3]), x);
+}
+
+template <int kVec, bool kNoise>
 __global__ __launch_bounds__(kSampThreads) void sampler_chunk_kernel(
     const bf16_t *__restrict__ logits, int64_t row_stride, const float *__restrict__ temperatures,
     const float *__restrict__ noise, int64_t noise_row_stride, uint64_t seed, uint64_t offset,
@@ -128,48 +154,33 @@ __global__ __launch_bounds__(kSampThreads) void sampler_chunk_kernel(
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(row) & 15u) == 0);
     const float t_in = temperatures[b];
     const bool greedy = (t_in == 0.f);
+    const int colbase = chunk * (kSampSlice * kVec) + tid * 8;      // slice v of this lane starts at colbase + v * kSampSlice
 
     // ---- every load of the chunk goes out before the first use ----------------------------------
-    u32x4_t raw[kSampVec];
-    int col0[kSampVec];
-    bool full[kSampVec];
+    u32x4_t raw[kVec];
 #pragma unroll
-    for (int v = 0; v < kSampVec; ++v) {
-        col0[v] = chunk * kSampChunk + v * kSampSlice + tid * 8;
-        full[v] = vec_ok && col0[v] + 8 <= vocab;
-        raw[v] = u32x4_t{0u, 0u, 0u, 0u};
-        if (full[v]) raw[v] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row + col0[v]));
-    }
-    float e[kSampVec][8];                                  // noise, where it is read
+    for (int v = 0; v < kVec; ++v) raw[v] = load_columns8(row, vec_ok, colbase + v * kSampSlice, vocab);
+    float e[kVec][8];                                      // noise, where it is read
     if (kNoise && !greedy) {
         const float *nrow = noise + static_cast<int64_t>(b) * noise_row_stride;
         const bool nvec_ok = ((reinterpret_cast<uintptr_t>(nrow) & 15u) == 0);
 #pragma unroll
-        for (int v = 0; v < kSampVec; ++v) {
-            if (nvec_ok && col0[v] + 8 <= vocab) {
-                const f32x4_t a = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(nrow + col0[v]));
-                const f32x4_t c = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(nrow + col0[v] + 4));
+        for (int v = 0; v < kVec; ++v) {
+            const int c0 = colbase + v * kSampSlice;
+            if (nvec_ok && c0 + 8 <= vocab) {
+                const f32x4_t a = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(nrow + c0));
+                const f32x4_t c = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(nrow + c0 + 4));
 #pragma unroll
                 for (int i = 0; i < 4; ++i) { e[v][i] = a[i]; e[v][4 + i] = c[i]; }
             } else {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) e[v][i] = (col0[v] + i < vocab) ? nrow[col0[v] + i] : 1.f;
+                for (int i = 0; i < 8; ++i) e[v][i] = (c0 + i < vocab) ? nrow[c0 + i] : 1.f;
             }
-        }
-    }
-    float x[kSampVec][8];                                  // columns past the row end read as -inf
-#pragma unroll
-    for (int v = 0; v < kSampVec; ++v) {
-        if (full[v]) {
-            unpack8(make_uint4(raw[v][0], raw[v][1], raw[v][2], raw[v][3]), x[v]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) x[v][i] = (col0[v] + i < vocab) ? bf16_to_f32(row[col0[v] + i]) : -INFINITY;
         }
     }
 
     __shared__ float sh_max[kSampWaves];
-    __shared__ float sh_sum[kSampWaves][kSampVec];
+    __shared__ float sh_sum[kSampWaves];
     __shared__ float sh_best[kSampWaves];
     __shared__ int sh_col[kSampWaves];
     SampRecord *rec = records + static_cast<int64_t>(b) * nchunks + chunk;
@@ -178,10 +189,14 @@ __global__ __launch_bounds__(kSampThreads) void sampler_chunk_kernel(
         float best = -INFINITY;
         int best_i = kNoToken;
 #pragma unroll
-        for (int v = 0; v < kSampVec; ++v)
+        for (int v = 0; v < kVec; ++v) {
+            float x[8];
+            const int c0 = colbase + v * kSampSlice;
+            columns8(raw[v], x);
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                if (col0[v] + i < vocab && x[v][i] > best) { best = x[v][i]; best_i = col0[v] + i; }
+                if (c0 + i < vocab && x[i] > best) { best = x[i]; best_i = c0 + i; }
+        }
         wave_best(best, best_i);
         if (lane == 0) { sh_best[wave] = best; sh_col[wave] = best_i; }
         __syncthreads();
@@ -192,110 +207,117 @@ __global__ __launch_bounds__(kSampThreads) void sampler_chunk_kernel(
         return;
     }
 
-    // ---- x / T (noise: the reference's division; otherwise folded into the base-2 exponent) ------
+    // ---- chunk maximum of x / T (noise: the reference's division; otherwise the scale is folded
+    //      into the base-2 exponent: y = x * log2(e) / T) ------------------------------------------
     const float k = 1.4426950408889634f / t_in;
     float m = -INFINITY;
+    float xt[kNoise ? kVec : 1][8];                        // noise: x / T, kept (8 values per lane); else recomputed from `raw`
 #pragma unroll
-    for (int v = 0; v < kSampVec; ++v)
+    for (int v = 0; v < kVec; ++v) {
+        float x[8];
+        columns8(raw[v], x);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            x[v][i] = kNoise ? x[v][i] / t_in : x[v][i] * k;
-            m = fmaxf(m, x[v][i]);
+            if (kNoise) {
+                xt[v][i] = x[i] / t_in;
+                m = fmaxf(m, xt[v][i]);
+            } else {
+                m = fmaxf(m, x[i] * k);
+            }
         }
+    }
     m = wave_max(m);
     if (lane == 0) sh_max[wave] = m;
     __syncthreads();
     m = fmaxf(fmaxf(sh_max[0], sh_max[1]), fmaxf(sh_max[2], sh_max[3]));
     const float mm = (m == -INFINITY) ? 0.f : m;           // a chunk of -inf logits: every weight is 0
+    if (!kNoise) forget(raw);
 
     if (kNoise) {
         float ssum = 0.f, best = -INFINITY;
         int best_i = kNoToken;
 #pragma unroll
-        for (int v = 0; v < kSampVec; ++v)
+        for (int v = 0; v < kVec; ++v) {
+            const int c0 = colbase + v * kSampSlice;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float ex = expf(x[v][i] - mm);       // exp(-inf) = 0 past the row end
+                const float ex = expf(xt[v][i] - mm);      // exp(-inf) = 0 past the row end
                 ssum += ex;
-                if (col0[v] + i < vocab) better(best, best_i, ex / fmaxf(e[v][i], 1e-10f), col0[v] + i);
+                if (c0 + i < vocab) better(best, best_i, ex / fmaxf(e[v][i], 1e-10f), c0 + i);
             }
+        }
         ssum = wave_sum(ssum);
         wave_best(best, best_i);
-        if (lane == 0) { sh_sum[wave][0] = ssum; sh_best[wave] = best; sh_col[wave] = best_i; }
+        if (lane == 0) { sh_sum[wave] = ssum; sh_best[wave] = best; sh_col[wave] = best_i; }
         __syncthreads();
         if (tid == 0) {
             for (int w = 1; w < kSampWaves; ++w) better(best, best_i, sh_best[w], sh_col[w]);
-            *rec = SampRecord{m, (sh_sum[0][0] + sh_sum[1][0]) + (sh_sum[2][0] + sh_sum[3][0]), best, best_i};
+            *rec = SampRecord{m, (sh_sum[0] + sh_sum[1]) + (sh_sum[2] + sh_sum[3]), best, best_i};
         }
         return;
     }
 
-    // ---- no noise tensor: weights, and the draw inside the chunk -----------------------------------
+    // ---- no noise tensor: the lane sums, and the draw inside the chunk -----------------------------
     // (the counter is wave-uniform, so the generator runs on the scalar unit beside the exponentials)
     const uint4 r = Philox::draw(make_uint4(static_cast<uint32_t>(b), 0x10000u + static_cast<uint32_t>(chunk),
                                             static_cast<uint32_t>(offset), static_cast<uint32_t>(offset >> 32)),
                                  make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)));
-    float part[kSampVec];                                  // this lane's 8-column sums, one per slice
+    float mine = 0.f;                                      // sum of this lane's weights, slice by slice, column by column
 #pragma unroll
-    for (int v = 0; v < kSampVec; ++v) {
-        float p = 0.f;
+    for (int v = 0; v < kVec; ++v) {
+        float x[8];
+        columns8(raw[v], x);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            x[v][i] = __builtin_amdgcn_exp2f(x[v][i] - mm);    // from here on x holds the weights
-            p += x[v][i];
-        }
-        part[v] = p;
+        for (int i = 0; i < 8; ++i) mine += __builtin_amdgcn_exp2f(x[i] * k - mm);    // exp2(-inf) = 0 past the row end
     }
-#pragma unroll
-    for (int v = 0; v < kSampVec; ++v) {
-        const float ws = wave_sum(part[v]);
-        if (lane == 0) sh_sum[wave][v] = ws;
-    }
+    const float wave_total = wave_sum(mine);
+    if (lane == 0) sh_sum[wave] = wave_total;
     __syncthreads();
-    float slice_sum[kSampVec];
-#pragma unroll
-    for (int v = 0; v < kSampVec; ++v) slice_sum[v] = (sh_sum[0][v] + sh_sum[1][v]) + (sh_sum[2][v] + sh_sum[3][v]);
-    const float chunk_sum = (slice_sum[0] + slice_sum[1]) + (slice_sum[2] + slice_sum[3]);
-    const int vsel = pick4(slice_sum, unit_uniform(r.x));                     // workgroup-uniform
-    if (vsel < 0) {                                        // no positive weight: the chunk can never be chosen
-        if (tid == 0) *rec = SampRecord{m, 0.f, 0.f, min(chunk * kSampChunk, vocab - 1)};
+    const float wsum[kSampWaves] = {sh_sum[0], sh_sum[1], sh_sum[2], sh_sum[3]};
+    const int wsel = pick4(wsum, unit_uniform(r.x));       // workgroup-uniform
+    if (wsel < 0) {                                        // no positive weight: the chunk can never be chosen
+        if (tid == 0) *rec = SampRecord{m, 0.f, 0.f, min(chunk * (kSampSlice * kVec), vocab - 1)};
         return;
     }
-    const float wsum[kSampWaves] = {sh_sum[0][vsel], sh_sum[1][vsel], sh_sum[2][vsel], sh_sum[3][vsel]};
-    const int wsel = pick4(wsum, unit_uniform(r.y));                          // > = 0: the slice has weight
     if (wave != wsel) return;                              // (wave-uniform; no barrier follows)
-    const float mine = vsel == 0 ? part[0] : vsel == 1 ? part[1] : vsel == 2 ? part[2] : part[3];
-    float incl = mine;                                     // inclusive scan over the 64 lanes
+    // ---- the chosen wavefront: which lane (inclusive scan of the 64 lane sums) -----------------
+    float incl = mine;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
         const float up = __shfl_up(incl, off, 64);
         if (lane >= off) incl += up;
     }
-    const double t3 = unit_uniform(r.z) * static_cast<double>(__shfl(incl, 63, 64));
+    const double t2 = unit_uniform(r.y) * static_cast<double>(__shfl(incl, 63, 64));
     const uint64_t live = __builtin_amdgcn_ballot_w64(mine > 0.f);            // != 0: the wavefront has weight
-    const uint64_t hit = __builtin_amdgcn_ballot_w64(mine > 0.f && static_cast<double>(incl) > t3);
+    const uint64_t hit = __builtin_amdgcn_ballot_w64(mine > 0.f && static_cast<double>(incl) > t2);
     const int lsel = hit != 0 ? __builtin_ctzll(hit) : 63 - __builtin_clzll(live);
-    if (lane != lsel) return;
-    float w8[8];
+    // ---- which of the lane's kVec * 8 columns: the lane hands its packed logits to the wavefront
+    //      through LDS and lane j recomputes the weight of the lane's j-th column (slice j / 8,
+    //      element j % 8), exactly as it was summed; one more scan instead of a serial walk --------
+    static_assert(kVec * 8 <= kWave, "one lane per column of the chosen lane");
+    __shared__ __attribute__((aligned(16))) uint32_t sh_cols[kVec * 4];
+    if (lane == lsel) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-        w8[i] = vsel == 0 ? x[0][i] : vsel == 1 ? x[1][i] : vsel == 2 ? x[2][i] : x[3][i];
-    float total = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) total += w8[i];
-    const double t4 = unit_uniform(r.w) * static_cast<double>(total);
-    float run = 0.f;
-    int isel = -1, ilive = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        run += w8[i];
-        if (w8[i] > 0.f) {
-            ilive = i;
-            if (isel < 0 && static_cast<double>(run) > t4) isel = i;
-        }
+        for (int v = 0; v < kVec; ++v) *reinterpret_cast<u32x4_t *>(&sh_cols[4 * v]) = raw[v];
     }
-    if (isel < 0) isel = ilive;
-    *rec = SampRecord{m, chunk_sum, 0.f, chunk * kSampChunk + vsel * kSampSlice + tid * 8 + isel};
+    __builtin_amdgcn_wave_barrier();                       // (one wavefront: its LDS accesses complete in order)
+    const int jj = lane < kVec * 8 ? lane : kVec * 8 - 1;
+    const uint32_t pair = sh_cols[jj >> 1];
+    const float xj = (jj & 1) ? bf16hi_to_f32(pair) : bf16lo_to_f32(pair);
+    const float wj = lane < kVec * 8 ? __builtin_amdgcn_exp2f(xj * k - mm) : 0.f;
+    float cincl = wj;
+#pragma unroll
+    for (int off = 1; off < kVec * 8; off <<= 1) {
+        const float up = __shfl_up(cincl, off, 64);
+        if (lane >= off) cincl += up;
+    }
+    const double t3 = unit_uniform(r.z) * static_cast<double>(__shfl(cincl, kVec * 8 - 1, 64));
+    const uint64_t clive = __builtin_amdgcn_ballot_w64(wj > 0.f);             // != 0: the lane has weight
+    const uint64_t chit = __builtin_amdgcn_ballot_w64(wj > 0.f && static_cast<double>(cincl) > t3);
+    const int jsel = chit != 0 ? __builtin_ctzll(chit) : 63 - __builtin_clzll(clive);
+    if (lane == 0)
+        *rec = SampRecord{m, (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]), 0.f,
+                          chunk * (kSampSlice * kVec) + (jsel >> 3) * kSampSlice + (wave * kWave + lsel) * 8 + (jsel & 7)};
 }
 
 // One wavefront per row: merges the row's chunk records into the token.
@@ -333,6 +355,36 @@ __global__ __launch_bounds__(kSampThreads) void sampler_row_kernel(
         return;
     }
     // ---- no noise tensor: the chunk is drawn by the chunk weights, the column inside it is in the record
+    const uint4 r = Philox::draw(make_uint4(static_cast<uint32_t>(b), 0x5a17u, static_cast<uint32_t>(offset),
+                                            static_cast<uint32_t>(offset >> 32)),
+                                 make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)));
+    if (nchunks <= kWave) {
+        // the usual case (vocabularies up to 524,288): one record per lane, read once, everything else in registers
+        SampRecord mine = SampRecord{-INFINITY, 0.f, 0.f, 0};
+        if (lane < nchunks) {
+            const f32x4_t v = *reinterpret_cast<const f32x4_t *>(rec + lane);
+            mine = SampRecord{v[0], v[1], v[2], __float_as_int(v[3])};
+        }
+        const float m = wave_max(mine.m);
+        if (m == -INFINITY) {                              // no finite logit in the row
+            if (lane == 0) out_tokens[b] = 0;
+            return;
+        }
+        const float w = mine.s * __builtin_amdgcn_exp2f(mine.m - m);      // 0 for lanes past the last chunk
+        double incl = static_cast<double>(w);
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const double up = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += up;
+        }
+        const double target = unit_uniform(r.x) * __shfl(incl, 63, 64);
+        const uint64_t live = __builtin_amdgcn_ballot_w64(w > 0.f);        // != 0: the row maximum's chunk has weight
+        const uint64_t hit = __builtin_amdgcn_ballot_w64(w > 0.f && incl > target);
+        const int pick = hit != 0 ? __builtin_ctzll(hit) : 63 - __builtin_clzll(live);
+        const int col = __shfl(mine.col, pick, 64);
+        if (lane == 0) out_tokens[b] = static_cast<int64_t>(col);
+        return;
+    }
     float m = -INFINITY;
     for (int c = lane; c < nchunks; c += kWave) m = fmaxf(m, rec[c].m);
     m = wave_max(m);
@@ -345,9 +397,6 @@ __global__ __launch_bounds__(kSampThreads) void sampler_row_kernel(
         total += static_cast<double>(rec[c].s * __builtin_amdgcn_exp2f(rec[c].m - m));
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) total += __shfl_xor(total, off, 64);
-    const uint4 r = Philox::draw(make_uint4(static_cast<uint32_t>(b), 0x5a17u, static_cast<uint32_t>(offset),
-                                            static_cast<uint32_t>(offset >> 32)),
-                                 make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)));
     const double target = unit_uniform(r.x) * total;
     double carry = 0.0;
     int pick = -1, last_live = -1;
@@ -374,12 +423,12 @@ __global__ __launch_bounds__(kSampThreads) void sampler_row_kernel(
 static int launch_sample(const bf16_t *logits, int64_t logits_row_stride, const float *temperatures,
                          const float *noise, int64_t noise_row_stride, uint64_t seed, uint64_t offset,
                          int64_t *out_tokens, SampRecord *records, int32_t batch, int32_t vocab, hipStream_t s) {
-    const int nchunks = samp_chunks(vocab);
+    const int nchunks = samp_chunks(vocab, noise ? kNoiseVec : kDrawVec);
     if (noise)
-        hipLaunchKernelGGL(sampler_chunk_kernel<true>, dim3(nchunks, batch), dim3(kSampThreads), 0, s, logits,
+        hipLaunchKernelGGL((sampler_chunk_kernel<kNoiseVec, true>), dim3(nchunks, batch), dim3(kSampThreads), 0, s, logits,
                            logits_row_stride, temperatures, noise, noise_row_stride, seed, offset, records, vocab, nchunks);
     else
-        hipLaunchKernelGGL(sampler_chunk_kernel<false>, dim3(nchunks, batch), dim3(kSampThreads), 0, s, logits,
+        hipLaunchKernelGGL((sampler_chunk_kernel<kDrawVec, false>), dim3(nchunks, batch), dim3(kSampThreads), 0, s, logits,
                            logits_row_stride, temperatures, noise, noise_row_stride, seed, offset, records, vocab, nchunks);
     if (launch_status() != NVA_OK) return NVA_ERR_LAUNCH_FAILED;
     hipLaunchKernelGGL(sampler_row_kernel, dim3((batch + kSampWaves - 1) / kSampWaves), dim3(kSampThreads), 0, s, records,
@@ -403,7 +452,8 @@ static int check_sample_args(const void *logits, int64_t logits_row_stride, cons
 
 extern "C" size_t nva_sample_workspace_bytes(int32_t batch, int32_t vocab) {
     if (batch <= 0 || vocab <= 0) return 0;
-    return static_cast<size_t>(batch) * nva::samp_chunks(vocab) * sizeof(nva::SampRecord);
+    // sized for the finer of the two chunkings (2048 columns, used when a noise tensor is given)
+    return static_cast<size_t>(batch) * nva::samp_chunks(vocab, nva::kNoiseVec) * sizeof(nva::SampRecord);
 }
 
 extern "C" int nva_sample(const void *logits, int64_t logits_row_stride, const float *temperatures,
@@ -467,7 +517,7 @@ extern "C" int nva_sample_static(const void *logits, int64_t logits_row_stride, 
     const int rc = check_sample_args(logits, logits_row_stride, temperatures, noise, noise_row_stride, out_tokens,
                                      batch, vocab);
     if (rc != NVA_OK || batch == 0) return rc;
-    if (static_cast<int64_t>(batch) * samp_chunks(vocab) > kStaticRecords) return NVA_ERR_SCRATCH_TOO_SMALL;
+    if (static_cast<int64_t>(batch) * samp_chunks(vocab, kNoiseVec) > kStaticRecords) return NVA_ERR_SCRATCH_TOO_SMALL;
     int status = NVA_OK;
     SampRecord *records = static_scratch(&status);
     if (records == nullptr) return status;

@@ -11,8 +11,9 @@
 // D*2 B written per tensor per stored token) and, at 4096 tokens, short enough that latency
 // decides: the row loads do not depend on the slot ids, so all of a lane's loads -- the slot ids
 // and kScatterTokens row chunks -- are issued together and only the stores wait for the slots
-// (rows whose slot turns out to be -1 are read in vain).  The cache rows are not read again by
-// this kernel: non-temporal stores.
+// (rows whose slot turns out to be -1 are read in vain).  Plain loads and stores: the rows were
+// just written by the producing kernel and are read next by the attention kernel, so both ends
+// profit from the caches (non-temporal loads measured 15 % slower, non-temporal stores equal).
 #include "nva_common.h"
 
 namespace nva {
@@ -40,11 +41,11 @@ __global__ __launch_bounds__(256) void store_kvcache_kernel(
         for (int t = 0; t < kScatterTokens; ++t) {
             const int64_t token = token0 + t < n_tokens ? token0 + t : n_tokens - 1;   // past the end: re-read the last row
             slot[t] = token0 + t < n_tokens ? slot_mapping[token] : -1;
-            row[t] = __builtin_nontemporal_load(src + token * stride + cc);
+            row[t] = src[token * stride + cc];
         }
 #pragma unroll
         for (int t = 0; t < kScatterTokens; ++t)      // -1 = skip (attention.py:22); never write out of bounds
-            if (slot[t] >= 0 && slot[t] < num_slots) __builtin_nontemporal_store(row[t], dst + slot[t] * chunks_per_row + cc);
+            if (slot[t] >= 0 && slot[t] < num_slots) dst[slot[t] * chunks_per_row + cc] = row[t];
     }
 }
 

@@ -15,8 +15,7 @@ bottom-right aligned causal mask when ``seqlen_k > seqlen_q`` (flash-attn >= 2.1
 softmax/accumulation and zero output for rows that see no keys.
 
 For draws without a noise tensor the library's own scheme is restated as well: a tree of
-inverse-CDF draws over the columns (``tree_draw``: row -> chunk -> slice -> group -> 8 columns ->
-column), every level with its own Philox4x32-10 uniform (``philox4x32_10``, ``row_uniforms``; pinned
+inverse-CDF draws (``tree_draw``: row -> chunk of 8192 columns -> column group -> lane -> column), every level with its own Philox4x32-10 uniform (``philox4x32_10``, ``row_uniforms``; pinned
 by the Random123 known-answer vectors), each level a walk through float64 running sums
 (``inverse_cdf_bounds`` is the one-level form).
 

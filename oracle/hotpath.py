@@ -238,11 +238,11 @@ def inverse_cdf_bounds(logits, temperatures):
     return p.cumsum(-1)
 
 
-# The library's draw without a noise tensor is a tree of such inverse-CDF draws over the columns in
-# column order, each level with its own uniform: row -> chunk of 8192 columns -> slice of 2048 ->
-# group of 512 -> group of 8 -> column.
+# The library's draw without a noise tensor is a tree of such inverse-CDF draws, each level with its
+# own uniform: row -> chunk of 8192 columns -> one of 4 column groups -> one of its 64 lanes -> one of
+# the lane's 32 columns.  Column ``2048 v + 512 g + 8 l + i`` of a chunk (v < 4, g < 4, l < 64, i < 8)
+# belongs to lane ``l`` of group ``g``; a lane's columns are walked in (v, i) order.
 TREE_CHUNK = 8192
-TREE_FANOUT = (4, 4, 64, 8)          # slices per chunk, groups per slice, 8-column groups per group, columns
 
 
 def _pick(weights, u):
@@ -267,17 +267,18 @@ def tree_draw(logits, temperatures, seed, offset):
     tensor -- the same distribution as nanovllm/layers/sampler.py:12-14, by other randomness.
 
     Row ``b`` picks a chunk of 8192 columns by the chunk weights with ``row_uniforms``; inside chunk
-    ``c`` the four output words of Philox counter ``(b, 0x10000 + c, offset)`` pick, in turn, one of
-    4 slices of 2048 columns, one of 4 groups of 512, one of 64 groups of 8 and one of 8 columns,
-    each by its share of the level's weight.  Returns ``(tokens int64 [B], margins float64 [B])``:
-    the margin is the smallest distance, over the levels, between a level's uniform and the edges
-    of the interval it fell into -- where it is tiny, fp32 sums may legitimately pick the neighbour.
+    ``c`` the first three output words of Philox counter ``(b, 0x10000 + c, offset)`` pick, in turn,
+    one of the 4 column groups, one of its 64 lanes and one of the lane's 32 columns, each by its
+    share of the level's weight.  Returns ``(tokens int64 [B], margins float64 [B])``: the margin is
+    the smallest distance, over the levels, between a level's uniform and the edges of the interval
+    it fell into -- where it is tiny, fp32 sums may legitimately pick the neighbour.
     A row without a finite logit yields token 0.
     """
     batch, vocab = logits.shape
     nchunks = -(-vocab // TREE_CHUNK)
     tokens = torch.zeros(batch, dtype=torch.int64)
     margins = torch.full((batch,), float("inf"), dtype=torch.float64)
+    cols = torch.arange(TREE_CHUNK).view(4, 4, 64, 8)                 # [v, group, lane, i] -> column inside the chunk
     for b in range(batch):
         y = logits[b].double() / float(temperatures[b])
         top = float(y.max())
@@ -287,13 +288,13 @@ def tree_draw(logits, temperatures, seed, offset):
         w[:vocab] = torch.exp(y - top)
         c, margin = _pick(w.view(nchunks, -1).sum(-1), _unit_uniform(_philox_words(seed, offset, b, 0x5A17)[0]))
         words = _philox_words(seed, offset, b, 0x10000 + c)
-        node, col = w[c * TREE_CHUNK:(c + 1) * TREE_CHUNK], c * TREE_CHUNK
-        for fan, word in zip(TREE_FANOUT, words):
-            node = node.view(fan, -1)
-            i, mg = _pick(node.sum(-1), _unit_uniform(word))
-            margin = min(margin, mg)
-            col += i * node.shape[1]
-            node = node[i]
-        tokens[b] = col
+        node = w[c * TREE_CHUNK:(c + 1) * TREE_CHUNK].view(4, 4, 64, 8)
+        g, mg = _pick(node.sum(dim=(0, 2, 3)), _unit_uniform(words[0]))
+        margin = min(margin, mg)
+        l, mg = _pick(node[:, g].sum(dim=(0, 2)), _unit_uniform(words[1]))
+        margin = min(margin, mg)
+        i, mg = _pick(node[:, g, l].reshape(32), _unit_uniform(words[2]))
+        margin = min(margin, mg)
+        tokens[b] = c * TREE_CHUNK + int(cols[:, g, l].reshape(32)[i])
         margins[b] = margin
     return tokens, margins

@@ -66,10 +66,10 @@ def test_store_kvcache_validation():
 def test_decode_validation_and_workspace_size():
     lib = _lib.load()
     ws = lib.nva_paged_decode_workspace_bytes
-    # prefix sums and context lengths (each 256-byte aligned) + a 32-byte record per worker +
-    # (2048 workers * min(heads, 8) + batch * heads) partial rows of 130 floats
-    assert ws(64, 16, 128, 8) == 512 + 256 + 2048 * 32 + (2048 * 8 + 64 * 16) * 130 * 4
-    assert ws(3, 2, 128, 1) == 256 + 256 + 2048 * 32 + (2048 * 2 + 3 * 2) * 130 * 4
+    # prefix sums and context lengths (each 256-byte aligned) + a 32-byte record per worker + 8 bytes per
+    # (sequence, head) pair (256-byte aligned) + (2048 workers * min(heads, 8) + batch * heads) partial rows of 130 floats
+    assert ws(64, 16, 128, 8) == 512 + 256 + 2048 * 32 + 64 * 16 * 8 + (2048 * 8 + 64 * 16) * 130 * 4
+    assert ws(3, 2, 128, 1) == 256 + 256 + 2048 * 32 + 256 + (2048 * 2 + 3 * 2) * 130 * 4
     assert ws(0, 16, 128, 8) == 0
     f = lib.nva_paged_decode_attn
     ok = dict(q=A, qs=2048, kc=A, vc=A, bt=A, bts=8, mb=8, cl=A, out=A, ws=A, wsb=ws(4, 16, 128, 8),
@@ -129,7 +129,7 @@ def test_prefill_validation():
 def test_sampler_validation_and_workspace_size():
     lib = _lib.load()
     ws = lib.nva_sample_workspace_bytes
-    assert ws(256, 151936) == 256 * 19 * 16 and ws(1, 1) == 16 and ws(2, 8193) == 64 and ws(0, 10) == 0   # one 16-byte record per 8192-column chunk
+    assert ws(256, 151936) == 256 * 75 * 16 and ws(1, 1) == 16 and ws(2, 2049) == 64 and ws(0, 10) == 0   # one 16-byte record per 2048-column chunk
     f = lib.nva_sample
     assert f(None, 100, A, None, 0, 0, 0, A, A, 1 << 20, 4, 100, None) == _lib.ERR_NULL_POINTER
     assert f(A, 100, A, None, 0, 0, 0, A, None, 1 << 20, 4, 100, None) == _lib.ERR_NULL_POINTER
@@ -186,5 +186,5 @@ def test_sample_static_validation():
     assert f(A, 99, A, None, 0, 0, 0, A, 4, 100, None) == _lib.ERR_BAD_STRIDE
     assert f(A, 100, A, None, 0, 0, 0, A, 4, 0, None) == _lib.ERR_BAD_SHAPE
     assert f(A, 100, A, None, 0, 0, 0, A, 0, 100, None) == _lib.OK
-    assert f(A, 151936, A, None, 0, 0, 0, A, 6899, 151936, None) == _lib.ERR_SCRATCH_TOO_SMALL    # 6899 * 19 records > 131072
-    assert f(A, 1 << 30, A, None, 0, 0, 0, A, 2, 1 << 30, None) == _lib.ERR_SCRATCH_TOO_SMALL     # 2 * 131072 records
+    assert f(A, 151936, A, None, 0, 0, 0, A, 1748, 151936, None) == _lib.ERR_SCRATCH_TOO_SMALL    # 1748 * 75 records > 131072
+    assert f(A, 1 << 29, A, None, 0, 0, 0, A, 1, 1 << 29, None) == _lib.ERR_SCRATCH_TOO_SMALL     # 262144 records

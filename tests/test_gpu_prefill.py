@@ -147,7 +147,10 @@ def test_prefill_sequences_do_not_leak(dev):
 def test_prefill_warmup_shape_4x4096(dev):
     """The runner's warm-up batch (4 sequences of max_model_len = 4096 tokens, packed, no cache):
     64 key tiles per row, far more than config 3 has.  One sequence is checked against the fp32
-    oracle in full; every sequence launched alone gives the same bits as inside the batch."""
+    oracle in full; every sequence launched alone, and the same four packed in another order, give
+    the same bits as inside the batch (a row's arithmetic does not depend on what else is in the
+    launch -- this is the check that catches a missed hardware wait state, which moves a result by
+    far less than the tolerance)."""
     g = torch.Generator().manual_seed(21)
     n, L = 4, 4096
     q = (torch.randn((n * L, 16, 128), generator=g)).to(torch.bfloat16)
@@ -163,7 +166,27 @@ def test_prefill_warmup_shape_4x4096(dev):
     want = oracle.varlen_prefill_attention(q[s * L:(s + 1) * L], k[s * L:(s + 1) * L], v[s * L:(s + 1) * L], one, one,
                                            scale, precision="fp32")
     assert_attn_close(out[s * L:(s + 1) * L], want, "4096-token sequence")
+    order = [2, 0, 3, 1]
+    pick = torch.cat([torch.arange(i * L, (i + 1) * L) for i in order]).to(dev)
+    again = varlen_prefill_attention(qd[pick], kd[pick], vd[pick], cu.to(dev), cu.to(dev), L, L, scale)
+    for j, i in enumerate(order):
+        assert torch.equal(bits(again[j * L:(j + 1) * L]), bits(out[i * L:(i + 1) * L]))
     for i in range(n):
         alone = varlen_prefill_attention(qd[i * L:(i + 1) * L], kd[i * L:(i + 1) * L], vd[i * L:(i + 1) * L],
                                          one.to(dev), one.to(dev), L, L, scale)
         assert torch.equal(bits(alone), bits(out[i * L:(i + 1) * L]))
+
+
+@pytest.mark.parametrize("hq,hkv,q_lens", [(4, 1, [4096, 300]), (16, 8, [2000, 100, 70, 1]), (2, 2, [1500])])
+def test_prefill_one_sequence_dominates(dev, hq, hkv, q_lens):
+    """Ragged batches in which one long sequence sits beside very short ones (query tiles of 2 to 64
+    key tiles in one launch), packed and through the block table, few heads and many."""
+    case = synthetic.prefill_case(seed=hq * 7, q_lens=q_lens, prefix_blocks=[0] * len(q_lens), num_heads=hq,
+                                  num_kv_heads=hkv, num_blocks=32)
+    out, want = _packed(case, dev)
+    assert_attn_close(out, want, "dominant sequence, packed")
+    prefix = [2] + [0] * (len(q_lens) - 1)
+    case = synthetic.prefill_case(seed=hq * 7 + 1, q_lens=q_lens, prefix_blocks=prefix, num_heads=hq, num_kv_heads=hkv,
+                                  num_blocks=40)
+    out, want = _paged(case, dev)
+    assert_attn_close(out, want, "dominant sequence, paged")

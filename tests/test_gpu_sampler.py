@@ -94,12 +94,13 @@ def test_sampler_philox_mode_is_categorical_and_reproducible(dev):
 
 
 @pytest.mark.parametrize("batch,vocab,scale", [(64, 151936, 2.0), (33, 4001, 1.0), (8, 50000, 4.0), (5, 7, 1.0),
-                                               (16, 8192, 1.0), (16, 8193, 3.0)])
+                                               (16, 8192, 1.0), (16, 8193, 3.0), (3, 8192 * 66 + 5, 2.0)])
 def test_sampler_in_kernel_draw_is_the_tree_of_inverse_cdf_draws(dev, batch, vocab, scale):
     """Without a noise tensor the token of row b is what the oracle's float64 tree of inverse-CDF
     draws yields from the same Philox uniforms.  The kernel sums in fp32, so rows whose uniform lies
     within rounding of an interval edge at some level may take the neighbouring branch; every other
-    row must agree exactly, and no row may return a column of zero probability."""
+    row must agree exactly, and no row may return a column of zero probability.  (The last case has
+    more than 64 chunks per row: the row kernel then walks the chunk records in several rounds.)"""
     g = torch.Generator().manual_seed(vocab)
     logits = (torch.randn(batch, vocab, generator=g) * scale).to(torch.bfloat16)
     logits[0, : min(3, vocab - 1)] = float("-inf")           # leading columns that cannot be drawn

@@ -345,7 +345,7 @@ def test_inverse_cdf_draws_the_softmax():
 
 def test_tree_draw_reduces_to_one_inverse_cdf_on_eight_columns():
     """With at most 8 columns only the last level of the tree has a choice, so the draw must be the
-    plain inverse CDF of that level's uniform: word 3 of Philox counter (row, 0x10000, offset)."""
+    plain inverse CDF of that level's uniform: word 2 of Philox counter (row, 0x10000, offset)."""
     g = torch.Generator().manual_seed(8)
     batch, seed, offset = 300, 0xABCDEF0123, 41
     logits = (torch.randn(batch, 8, generator=g) * 1.5).to(torch.bfloat16)
@@ -353,7 +353,7 @@ def test_tree_draw_reduces_to_one_inverse_cdf_on_eight_columns():
     temps = torch.linspace(0.4, 1.6, batch)
     tok, margin = oracle.tree_draw(logits, temps, seed, offset)
     bounds = oracle.inverse_cdf_bounds(logits, temps)
-    u = torch.tensor([(oracle.philox4x32_10((b, 0x10000, offset, 0), (seed & 0xFFFFFFFF, seed >> 32))[3] + 0.5) * 2.0 ** -32
+    u = torch.tensor([(oracle.philox4x32_10((b, 0x10000, offset, 0), (seed & 0xFFFFFFFF, seed >> 32))[2] + 0.5) * 2.0 ** -32
                       for b in range(batch)], dtype=torch.float64)
     want = torch.searchsorted(bounds, u.unsqueeze(1), right=True).squeeze(1)
     sure = margin > 1e-9
@@ -362,9 +362,9 @@ def test_tree_draw_reduces_to_one_inverse_cdf_on_eight_columns():
 
 
 def test_tree_draw_is_categorical_across_all_levels():
-    """Heavy columns placed so that every level of the tree has to choose (different chunks, slices,
-    groups of 512, groups of 8 and neighbours inside a group of 8): empirical frequencies over many
-    rows against softmax(logits / T), chi-square."""
+    """Heavy columns placed so that every level of the tree has to choose (different chunks, column
+    groups, lanes, and columns of one lane in the same and in different 2048-column slices):
+    empirical frequencies over many rows against softmax(logits / T), chi-square."""
     cols = [3, 5, 6, 11, 700, 2050, 2051, 4100, 8191, 8192, 9000, 16390, 19999]
     vocab, n, t = 20000, 12000, 0.9
     row = torch.full((vocab,), float("-inf"))

@@ -43,7 +43,7 @@ def _both(dev, batch, vocab, with_noise, seed, offset, temperature=0.6):
 
 @pytest.mark.parametrize("with_noise", [False, True])
 def test_sample_static_matches_sample_on_two_calls_in_a_row(dev, with_noise):
-    big = _both(dev, 256, 151936, with_noise, seed=17, offset=3)          # 256 x 19 records of the scratch array
+    big = _both(dev, 256, 151936, with_noise, seed=17, offset=3)          # up to 256 x 75 records of the scratch array
     small = _both(dev, 7, 5000, with_noise, seed=17, offset=4)            # then 7 records: stale ones beyond must not matter
     again = _both(dev, 256, 151936, with_noise, seed=17, offset=3)
     assert torch.equal(big, again) and small.numel() == 7
@@ -51,7 +51,7 @@ def test_sample_static_matches_sample_on_two_calls_in_a_row(dev, with_noise):
 
 def test_sample_static_rejects_what_does_not_fit(dev):
     lib = _lib.load()
-    batch, vocab = 6899, 151936                                           # 6899 * 19 records > 131072
+    batch, vocab = 1748, 151936                                           # 1748 * 75 records > 131072
     out = torch.full((4,), -5, dtype=torch.int64, device=dev)
     rc = lib.nva_sample_static(0x1000, vocab, 0x1000, None, 0, 0, 0, out.data_ptr(), batch, vocab,
                                torch.cuda.current_stream().cuda_stream)
