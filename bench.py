@@ -202,11 +202,11 @@ def bench_sampler(args, dev):
     result = {
         "metric": "sampler (in-kernel randomness), achieved HBM GB/s", "value": round(gbps, 1), "unit": "GB/s",
         "ms_per_step": round(per_step_ms, 5),
-        "config": {"workload": "sampler: 256 rows x 151,936 bf16 logits, T=0.6, in-kernel randomness (one uniform per row, inverse CDF)",
+        "config": {"workload": "sampler: 256 rows x 151,936 bf16 logits, T=0.6, in-kernel randomness (tree of inverse-CDF draws, Philox uniforms)",
                    "batch": batch},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "sampler_cdf_sums_kernel + sampler_cdf_select_kernel",
+                     "kernel": "sampler_chunk_kernel<4, false> + sampler_row_kernel",
                      "algorithmic_bytes_per_launch": alg},
     }
 
@@ -420,7 +420,7 @@ def bench_e2e(args, dev):
     from nanovllm_amd.engine import SamplingParams, qwen3_0_6b
     from nanovllm_amd.engine.llm import LLM
     model = qwen3_0_6b()
-    llm = LLM(model, enforce_eager=args.eager, max_model_len=4096, num_kvcache_blocks=4096)
+    llm = LLM(model, enforce_eager=args.eager, max_model_len=4096, num_kvcache_blocks=4096, graph_bucket_step=args.bucket_step)
     prompts, params = e2e_workload(num_seqs=args.requests, max_output_len=args.max_output_len)
     total_out = sum(p.max_tokens for p in params)
     llm.generate([[1, 2, 3, 4]], SamplingParams(max_tokens=8, ignore_eos=True))     # reference warm-up call
@@ -432,6 +432,9 @@ def bench_e2e(args, dev):
     layers = [m for m in llm.model_runner.model.modules() if isinstance(m, nva.Attention)]
     roof = decode_e2e_shape_roofline(dev, [(a.k_cache, a.v_cache) for a in layers], llm.config.num_kvcache_blocks)
     st = dict(llm.stats)
+    used, replayed = llm.model_runner.bucket_rows
+    buckets = {"graph_bucket_step": llm.config.graph_bucket_step, "decode_rows_used": used, "decode_rows_replayed": replayed,
+               "padded_fraction": round(1 - used / max(replayed, 1), 4)}
     del layers, llm
     gc.collect()
     torch.cuda.empty_cache()
@@ -443,7 +446,8 @@ def bench_e2e(args, dev):
                                "U[100,1024], temperature 0.6, ignore_eos, prompt ids drawn afresh for every pass, "
                                + ("eager" if args.eager else "hipGraph decode"),
                    "requests": args.requests, "output_tokens": total_out, "engine_steps_per_pass": (st["prefill_steps"] + st["decode_steps"]) // args.steps,
-                   "prefill_s_per_pass": round(st["prefill_s"] / args.steps, 3), "decode_s_per_pass": round(st["decode_s"] / args.steps, 3)},
+                   "prefill_s_per_pass": round(st["prefill_s"] / args.steps, 3), "decode_s_per_pass": round(st["decode_s"] / args.steps, 3),
+                   "decode_buckets": buckets},
         "roofline": roof,
     }
     if not args.no_extra:
@@ -558,6 +562,7 @@ def main():
     ap.add_argument("--requests", type=int, default=256, help="e2e only: number of requests (profiling runs)")
     ap.add_argument("--max-output-len", type=int, default=1024, help="e2e only: cap on output lengths (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--bucket-step", type=int, default=16, help="e2e only: spacing of the captured decode batch sizes")
     ap.add_argument("--no-extra", action="store_true", help="e2e only: skip the per-configuration rooflines and the eager pass")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -61,6 +61,7 @@ def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor,
 
 
 _workspaces: dict = {}
+_retired_workspaces: list = []
 
 
 def _decode_workspace(device, nbytes: int) -> torch.Tensor:
@@ -70,11 +71,15 @@ def _decode_workspace(device, nbytes: int) -> torch.Tensor:
     only grows outside graph capture: a captured graph
     must be preceded by an eager warm-up call of the same shape, which is what the runner
     does before capturing each batch size (nanovllm/engine/model_runner.py:232-234).
+    A buffer that is replaced by a larger one is kept alive until the process ends: graphs
+    captured earlier (and the work split they reuse) hold its address.
     """
     ws = _workspaces.get(device)
     if ws is None or ws.numel() < nbytes:
         if torch.cuda.is_current_stream_capturing():
             raise RuntimeError("decode workspace must be allocated by an eager warm-up call before graph capture")
+        if ws is not None:
+            _retired_workspaces.append(ws)
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[device] = ws
     return ws

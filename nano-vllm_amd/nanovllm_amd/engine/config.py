@@ -70,6 +70,7 @@ class EngineConfig:
     num_kvcache_blocks: int = -1
     seed: int = 0
     decode_lookahead: bool = True                        # launch decode steps one step ahead of their tokens
+    graph_bucket_step: int = 16                          # decode graphs are captured for batch sizes 1, 2, 4, 8 and every multiple of this
 
     def __post_init__(self):
         if isinstance(self.model, ModelConfig):
@@ -80,5 +81,6 @@ class EngineConfig:
         assert self.kvcache_block_size % 256 == 0
         assert self.kvcache_block_size == 256, "the attention kernels are built for 256-token KV blocks"
         assert self.tensor_parallel_size == 1, "this build runs on one GPU"
+        assert self.graph_bucket_step >= 1
         self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
         assert self.max_num_batched_tokens >= self.max_model_len

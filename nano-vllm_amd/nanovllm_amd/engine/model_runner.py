@@ -108,6 +108,7 @@ class ModelRunner:
         self.max_table_width = -(-config.max_model_len // self.block_size)
         self.graphs = {}
         self.graph_bs: List[int] = []
+        self.bucket_rows = [0, 0]                        # decode rows used / rows replayed (bucket padding), since start
         self.graph_segments = 4                          # consecutive graphs per decode step (see capture_graphs)
         self._graph_keepalive = []
         with torch.inference_mode():
@@ -157,13 +158,49 @@ class ModelRunner:
     def prepare_block_tables(self, seqs: List[Sequence]) -> torch.Tensor:
         return self._to_device(build_block_tables(seqs), torch.int32)
 
+    def _init_prefill_staging(self) -> None:
+        """Pinned host buffers (two, used in turn) and one device buffer for everything a prefill step
+        needs on the device: the step's arrays are packed one after the other and cross PCIe in a
+        single kernel (the reference issues one pinned copy per tensor, nanovllm/engine/
+        model_runner.py:155-159,184)."""
+        cfg = self.config
+        tokens, seqs = cfg.max_num_batched_tokens, cfg.max_num_seqs
+        total = tokens * (8 + 8 + 4) + 2 * (seqs + 1) * 4 + seqs * self.max_table_width * 4 + seqs * 4 + 8 * 256
+        self._pf_host = [torch.zeros(total, dtype=torch.uint8).pin_memory() for _ in range(2)]
+        self._pf_dev = torch.zeros(total, dtype=torch.uint8, device=self.device)
+        self._pf_turn = 0
+
+    def _stage_prefill(self, fields):
+        """``fields``: list of (numpy array, torch dtype).  Packs them (256-byte aligned) into a pinned
+        buffer, copies the used part to the device with one kernel and returns device views."""
+        if not hasattr(self, "_pf_host"):
+            self._init_prefill_staging()
+        self._pf_turn ^= 1
+        host = self._pf_host[self._pf_turn].numpy()
+        at, views = 0, []
+        for array, dtype in fields:
+            if array is None:
+                views.append(None)
+                continue
+            raw = np.ascontiguousarray(array).view(np.uint8).reshape(-1)
+            if at + raw.size > host.size:
+                raise RuntimeError("prefill step exceeds max_num_batched_tokens / max_num_seqs")
+            host[at: at + raw.size] = raw
+            views.append(self._pf_dev[at: at + raw.size].view(dtype).view(array.shape))
+            at += (raw.size + 255) // 256 * 256
+        rc = _lib.load().nva_stage_decode_inputs(self._pf_dev.data_ptr(), self._pf_host[self._pf_turn].data_ptr(), at,
+                                                 0, 0, 0, None, 0, torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "nva_stage_decode_inputs")
+        return views
+
     def prepare_prefill(self, seqs: List[Sequence]):
         h = build_prefill_inputs(seqs, self.block_size)
-        block_tables = self._to_device(h["block_tables"], torch.int32) if h["block_tables"] is not None else None
-        set_context(True, self._to_device(h["cu_seqlens_q"], torch.int32), self._to_device(h["cu_seqlens_k"], torch.int32),
-                    h["max_seqlen_q"], h["max_seqlen_k"], self._to_device(h["slot_mapping"], torch.int32), None,
-                    block_tables)
-        return self._to_device(h["input_ids"], torch.int64), self._to_device(h["positions"], torch.int64)
+        ids, pos, cu_q, cu_k, slots, tables, self._pf_temperatures = self._stage_prefill([
+            (h["input_ids"], torch.int64), (h["positions"], torch.int64), (h["cu_seqlens_q"], torch.int32),
+            (h["cu_seqlens_k"], torch.int32), (h["slot_mapping"], torch.int32), (h["block_tables"], torch.int32),
+            (np.fromiter((s.temperature for s in seqs), dtype=np.float32, count=len(seqs)), torch.float32)])
+        set_context(True, cu_q, cu_k, h["max_seqlen_q"], h["max_seqlen_k"], slots, None, tables)
+        return ids, pos
 
     def prepare_decode(self, seqs: List[Sequence]):
         h = build_decode_inputs(seqs, self.block_size)
@@ -211,6 +248,8 @@ class ModelRunner:
         whose last token is still pending take it on the device from ``prev``'s sampler output."""
         bs = len(seqs)
         bucket = next(x for x in self.graph_bs if x >= bs)
+        self.bucket_rows[0] += bs                                 # rows that carry a sequence / rows replayed
+        self.bucket_rows[1] += bucket
         h = build_decode_inputs(seqs, self.block_size)
         self._stage_turn ^= 1
         st = self._stage_np[self._stage_turn]
@@ -271,8 +310,12 @@ class ModelRunner:
                 logits = self._run_decode_graph(seqs)
                 temperatures = self.graph_vars["temperatures"][: len(seqs)]
             else:
-                input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
-                temperatures = self.prepare_sample(seqs)
+                if is_prefill:
+                    input_ids, positions = self.prepare_prefill(seqs)
+                    temperatures = self._pf_temperatures          # staged with the other prefill inputs
+                else:
+                    input_ids, positions = self.prepare_decode(seqs)
+                    temperatures = self.prepare_sample(seqs)
                 logits = self.run_model(input_ids, positions, is_prefill)
             tokens = self.sampler(logits, temperatures).tolist()   # the one device->host sync per step
         reset_context()
@@ -287,7 +330,10 @@ class ModelRunner:
         input_ids, positions, slot_mapping = gv["input_ids"], gv["positions"], gv["slot_mapping"]
         context_lens, block_tables = gv["context_lens"], gv["block_tables"]
         outputs = torch.zeros(max_bs, self.cfg.hidden_size, dtype=torch.bfloat16, device=self.device)
-        self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))
+        step = cfg.graph_bucket_step                      # the reference captures 1, 2, 4, 8 and every 16th size (model_runner.py:227)
+        self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs and b < step] + list(range(step, max_bs + 1, step))
+        if self.graph_bs[-1] != max_bs:
+            self.graph_bs.append(max_bs)
         # The layer stack of a bucket is captured as several consecutive graphs instead of one:
         # launching a graph costs the host about a microsecond per node before the first kernel
         # starts, and with segments only the first segment's launch is exposed -- the others are
