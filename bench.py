@@ -10,7 +10,8 @@ already resident in HBM.  Workloads (shapes are the five benchmark configuration
     decode    paged decode attention, batch 64, 16/8 heads, ctx U[100,2048]       (config 2)
     scatter   store_kvcache, 4096 tokens into 512 blocks x 256 slots              (config 1)
     prefill   causal varlen prefill, 16 sequences, half with cached prefix        (config 3)
-    sampler   temperature sampling over 256 x 151,936 logits
+    sampler   temperature sampling over 256 x 151,936 logits (--noise: the replayable path with an Exp(1) tensor)
+    rope-scatter  q/k norm + rotary + cache write in one kernel, 16,384 tokens (the scatter the engine runs)
     decode-e2e-shape / decode-longctx-shape / copy   profiling helpers: the decode attention of configs 4 / 5
               alone (one layer); a plain copy of known size
 The line carries `roofline` (algorithmic bytes or flops of the dominant kernel per launch,
@@ -118,8 +119,9 @@ def bench_scatter(args, dev):
     from nanovllm_amd import synthetic
     pools = 4
     fns, alg, cases = [], [], []
+    n_tokens = getattr(args, "tokens", None) or 4096
     for p in range(pools):
-        c = synthetic.scatter_case(seed=p)
+        c = synthetic.scatter_case(seed=p, n_tokens=n_tokens)
         k, v, kc, vc, sm = (t.to(dev) for t in (c.key, c.value, c.k_cache, c.v_cache, c.slot_mapping))
         cases.append(c)
         alg.append(c.algorithmic_bytes)
@@ -130,8 +132,8 @@ def bench_scatter(args, dev):
     result = {
         "metric": "store_kvcache, achieved HBM GB/s (config 1)", "value": round(gbps, 1), "unit": "GB/s",
         "ms_per_step": round(per_step_ms, 5),
-        "config": {"workload": "store_kvcache config1: 4096 tokens x 8 kv heads x 128, 512 blocks x 256 slots, "
-                               "5% skipped", "tokens": 4096},
+        "config": {"workload": "store_kvcache config1: %d tokens x 8 kv heads x 128, 512 blocks x 256 slots, "
+                               "5%% skipped" % n_tokens, "tokens": n_tokens},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "store_kvcache_kernel",
                      "algorithmic_bytes_per_launch": int(alg[0])},
@@ -194,19 +196,25 @@ def bench_sampler(args, dev):
         logits = (torch.randn((batch, vocab), generator=g, device=dev) * 2).to(torch.bfloat16)
         sets.append(logits)
     temps = torch.full((batch,), 0.6, device=dev)
-    fns = [lambda l=l, i=i: nva.sample(l, temps, None, seed=1, offset=i) for i, l in enumerate(sets)]
+    with_noise = bool(getattr(args, "noise", False))
+    if with_noise:                                   # the replayable path: an Exp(1) tensor per set of logits is read as well
+        noises = [torch.empty((batch, vocab), device=dev).exponential_(1.0, generator=g) for _ in sets]
+        fns = [lambda l=l, n=n: nva.sample(l, temps, n) for l, n in zip(sets, noises)]
+    else:
+        fns = [lambda l=l, i=i: nva.sample(l, temps, None, seed=1, offset=i) for i, l in enumerate(sets)]
     ms = _event_time_ms(fns, args.steps, args.warmup)
     per_step_ms = ms / args.steps
-    alg = batch * vocab * 2
+    alg = batch * vocab * (6 if with_noise else 2)
     gbps = alg / (per_step_ms * 1e-3) / 1e9
     result = {
-        "metric": "sampler (in-kernel randomness), achieved HBM GB/s", "value": round(gbps, 1), "unit": "GB/s",
+        "metric": "sampler (%s), achieved HBM GB/s" % ("noise tensor given" if with_noise else "in-kernel randomness"),
+        "value": round(gbps, 1), "unit": "GB/s",
         "ms_per_step": round(per_step_ms, 5),
         "config": {"workload": "sampler: 256 rows x 151,936 bf16 logits, T=0.6, in-kernel randomness (tree of inverse-CDF draws, Philox uniforms)",
                    "batch": batch},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "sampler_chunk_kernel<4, false> + sampler_row_kernel",
+                     "kernel": ("sampler_chunk_kernel<1, true>" if with_noise else "sampler_chunk_kernel<4, false>") + " + sampler_row_kernel",
                      "algorithmic_bytes_per_launch": alg},
     }
 
@@ -220,6 +228,38 @@ def bench_sampler(args, dev):
                 "kind": "port", "sample": "64 of the 256 rows, eager torch sampler with pre-drawn noise, "
                                           "median of 5", "seconds": round(sec, 4)}
     return result, cpu
+
+
+def bench_rope_scatter(args, dev):
+    """The scatter as the engine runs it: q/k norm + rotary embedding + cache write in one kernel
+    (nva_qk_norm_rope with cache pointers), Qwen3-0.6B head geometry, a prefill-sized batch of tokens."""
+    import torch
+    from nanovllm_amd.engine import layers
+    n, hq, hkv, d = (getattr(args, "tokens", None) or 16384), 16, 8, 128
+    g = torch.Generator(device=dev).manual_seed(1)
+    w = torch.ones(d, dtype=torch.bfloat16, device=dev)
+    rope = layers.build_rope_cache(d, 4096, 1e6, dev)
+    pos = torch.randint(0, 4096, (n,), device=dev)
+    fns = []
+    for p in range(3):
+        qkv = torch.randn(n, (hq + 2 * hkv) * d, device=dev, generator=g).to(torch.bfloat16)
+        kc = torch.zeros(512, 256, hkv, d, dtype=torch.bfloat16, device=dev)
+        vc = torch.zeros_like(kc)
+        sm = torch.randperm(131072, device=dev)[:n].to(torch.int32)
+        fns.append(lambda qkv=qkv, kc=kc, vc=vc, sm=sm: layers.qk_norm_rope(qkv, pos, w, w, rope, hq, hkv, d, 1e-6,
+                                                                            kv_store=(kc, vc, sm)))
+    ms = _event_time_ms(fns, args.steps, args.warmup) / args.steps
+    # per token: the qkv row in; q, k out; the K and V cache rows out; one rope table row, a position and a slot id in
+    alg = n * ((hq + 2 * hkv) * d * 2 + (hq + hkv) * d * 2 + 2 * hkv * d * 2 + d * 4 + 8 + 4)
+    gbps = alg / (ms * 1e-3) / 1e9
+    result = {"metric": "q/k norm + rotary + KV-cache scatter in one kernel, achieved HBM GB/s", "value": round(gbps, 1),
+              "unit": "GB/s", "ms_per_step": round(ms, 5),
+              "config": {"workload": "nva_qk_norm_rope with cache pointers: %d tokens, 16q/8kv heads x 128, slots drawn from "
+                                     "512 blocks x 256" % n, "tokens": n},
+              "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "qk_norm_rope_kernel",
+                           "algorithmic_bytes_per_launch": alg}}
+    return result, (lambda: None)
 
 
 def e2e_workload(num_seqs=256, max_input_len=1024, max_output_len=1024, vocab=151936, seed=0):
@@ -391,10 +431,12 @@ def collect_extra(dev, model, prompts, params):
     from types import SimpleNamespace
     from nanovllm_amd.engine.llm import LLM
     extra = {}
-    for name, fn, steps in (("scatter_config1", bench_scatter, 400), ("decode_config2", bench_decode, 112),
-                            ("prefill_config3", bench_prefill, 50), ("sampler_256x151936", bench_sampler, 100),
-                            ("decode_config5_shape", bench_decode_longctx_shape, 1)):
-        result, _ = fn(SimpleNamespace(steps=steps, warmup=max(3, steps // 10)), dev)
+    for name, fn, steps, kw in (("scatter_config1", bench_scatter, 400, {}), ("rope_scatter_16384_tokens", bench_rope_scatter, 100, {}),
+                                ("decode_config2", bench_decode, 112, {}), ("prefill_config3", bench_prefill, 50, {}),
+                                ("sampler_256x151936", bench_sampler, 100, {}),
+                                ("sampler_with_noise_256x151936", bench_sampler, 50, {"noise": True}),
+                                ("decode_config5_shape", bench_decode_longctx_shape, 1, {})):
+        result, _ = fn(SimpleNamespace(steps=steps, warmup=max(3, steps // 10), **kw), dev)
         extra[name] = dict(result["roofline"], us_per_launch=round(result["ms_per_step"] * 1e3, 2))
         del result
         gc.collect()
@@ -547,9 +589,9 @@ def bench_longctx(args, dev):
     return result, (lambda: None)
 
 
-WORKLOADS = {"e2e": bench_e2e, "longctx": bench_longctx, "decode-e2e-shape": bench_decode_e2e_shape,
+WORKLOADS = {"rope-scatter": bench_rope_scatter, "e2e": bench_e2e, "longctx": bench_longctx, "decode-e2e-shape": bench_decode_e2e_shape,
              "decode-longctx-shape": bench_decode_longctx_shape, "copy": bench_copy, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
-DEFAULT_STEPS = {"e2e": 1, "longctx": 1, "decode-e2e-shape": 1, "decode-longctx-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
+DEFAULT_STEPS = {"rope-scatter": 100, "e2e": 1, "longctx": 1, "decode-e2e-shape": 1, "decode-longctx-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
 
 
 def main():
@@ -562,6 +604,8 @@ def main():
     ap.add_argument("--requests", type=int, default=256, help="e2e only: number of requests (profiling runs)")
     ap.add_argument("--max-output-len", type=int, default=1024, help="e2e only: cap on output lengths (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--tokens", type=int, default=None, help="scatter / rope-scatter: number of tokens (default 4096 / 16384)")
+    ap.add_argument("--noise", action="store_true", help="sampler: time the replayable path that reads an Exp(1) noise tensor")
     ap.add_argument("--bucket-step", type=int, default=16, help="e2e only: spacing of the captured decode batch sizes")
     ap.add_argument("--no-extra", action="store_true", help="e2e only: skip the per-configuration rooflines and the eager pass")
     args = ap.parse_args()

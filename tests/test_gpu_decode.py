@@ -240,3 +240,31 @@ def test_decode_config5_full_size(dev):
     del out2
     ones = paged_decode_attention(q.to(dev), kc, torch.ones_like(vc), ctx.to(dev), tables.to(dev), scale)
     assert (ones.float() - 1).abs().max().item() < 1e-2
+
+
+@pytest.mark.parametrize("batch,hq,hkv", [(32, 16, 8), (31, 16, 8), (64, 32, 8), (40, 8, 8), (300, 16, 8), (33, 8, 8)])
+def test_decode_ragged_batches_share_a_workspace(dev, batch, hq, hkv):
+    """Ragged contexts with empty, one-token and very short sequences beside long ones, batch sizes
+    from few to many (sequence, kv head) pairs per worker, several decode steps in a row on the one
+    workspace of the device (a build and two reuses of the work split each), against the fp32
+    oracle; every call of a geometry returns the same bits."""
+    g = torch.Generator().manual_seed(batch * 100 + hq)
+    lens = torch.randint(1, 3000, (batch,), generator=g)
+    lens[::7] = torch.randint(1, 40, (len(lens[::7]),), generator=g)          # very short ones
+    lens[3] = 0
+    lens[5] = 1
+    need = int(((lens + 255) // 256).sum()) + 4
+    case = synthetic.decode_case(seed=batch + hq, num_heads=hq, num_kv_heads=hkv, num_blocks=need, context_lens=lens.tolist())
+    want = _oracle(case)
+    q, kc, vc, cl, bt = (t.to(dev) for t in (case.q, case.k_cache, case.v_cache, case.context_lens, case.block_tables))
+    outs = []
+    for _ in range(3):
+        plan = DecodePlan()
+        for _layer in range(3):                                  # one build, two reuses
+            outs.append(paged_decode_attention(q, kc, vc, cl, bt, case.scale, plan=plan).clone())
+    torch.cuda.synchronize()
+    for o in outs:
+        assert_attn_close(o, want, f"batch {batch}")
+    for o in outs[1:]:
+        assert torch.equal(bits(o), bits(outs[0]))
+    assert not outs[0][3].any()
