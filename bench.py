@@ -120,8 +120,11 @@ def bench_scatter(args, dev):
     pools = 4
     fns, alg, cases = [], [], []
     n_tokens = getattr(args, "tokens", None) or 4096
+    contiguous = bool(getattr(args, "contiguous", False))
     for p in range(pools):
         c = synthetic.scatter_case(seed=p, n_tokens=n_tokens)
+        if contiguous:                               # slots as a prefill produces them: runs of consecutive slots, block by block
+            c.slot_mapping = torch.where(c.slot_mapping >= 0, c.slot_mapping.sort().values, c.slot_mapping)
         k, v, kc, vc, sm = (t.to(dev) for t in (c.key, c.value, c.k_cache, c.v_cache, c.slot_mapping))
         cases.append(c)
         alg.append(c.algorithmic_bytes)
@@ -133,7 +136,7 @@ def bench_scatter(args, dev):
         "metric": "store_kvcache, achieved HBM GB/s (config 1)", "value": round(gbps, 1), "unit": "GB/s",
         "ms_per_step": round(per_step_ms, 5),
         "config": {"workload": "store_kvcache config1: %d tokens x 8 kv heads x 128, 512 blocks x 256 slots, "
-                               "5%% skipped" % n_tokens, "tokens": n_tokens},
+                               "5%% skipped%s" % (n_tokens, ", slots in ascending order" if contiguous else ""), "tokens": n_tokens},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "store_kvcache_kernel",
                      "algorithmic_bytes_per_launch": int(alg[0])},
@@ -605,6 +608,7 @@ def main():
     ap.add_argument("--max-output-len", type=int, default=1024, help="e2e only: cap on output lengths (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--tokens", type=int, default=None, help="scatter / rope-scatter: number of tokens (default 4096 / 16384)")
+    ap.add_argument("--contiguous", action="store_true", help="scatter: slots in ascending order instead of a random permutation")
     ap.add_argument("--noise", action="store_true", help="sampler: time the replayable path that reads an Exp(1) noise tensor")
     ap.add_argument("--bucket-step", type=int, default=16, help="e2e only: spacing of the captured decode batch sizes")
     ap.add_argument("--no-extra", action="store_true", help="e2e only: skip the per-configuration rooflines and the eager pass")

@@ -234,6 +234,8 @@ int nva_rms_norm(const void *x, int64_t x_row_stride,
  * [num_slots, num_kv_heads * head_dim] and int32 [n_tokens] slots: the rotated key row and the
  * (unchanged) value row of token i are also written to cache row slot_mapping[i], bit-identical
  * to what nva_store_kvcache would write from k_out and the v view; -1 / out-of-range skips.
+ * Every tensor pointer must be 16-byte aligned and qkv_row_stride a multiple of 8 elements
+ * (NVA_ERR_MISALIGNED / NVA_ERR_BAD_STRIDE otherwise): all accesses are 16 bytes per lane.
  */
 int nva_qk_norm_rope(const void *qkv, int64_t qkv_row_stride, const int64_t *positions,
                      const void *q_weight, const void *k_weight, const float *rope_cache,

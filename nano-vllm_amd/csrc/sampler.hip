@@ -11,8 +11,9 @@
 //
 // With a caller-supplied tensor of E ~ Exp(1) draws (replayable; used for parity; chunks of 2048
 // columns) the score of column i is evaluated relative to the CHUNK maximum m_c,
-// e_i = exp(x_i - m_c) / max(E_i, 1e-10) with the reference's true fp32 division by T, and the
-// record keeps (m_c, sum exp, best e_i, its column).  The row merge scales every chunk's best by
+// e_i = exp(x_i - m_c) / max(E_i, 1e-10), and the record keeps (m_c, sum exp, best e_i, its column).
+// The two divisions per column (by T and by the noise) are a multiplication by 1/T and by a
+// one-ulp hardware reciprocal: true fp32 divisions made this pass instruction-bound.  The row merge scales every chunk's best by
 // exp(m_c - M) / S: the same quantity softmax(x)_i / E_i the reference maximises, factored as
 // exp(x_i - m_c) * exp(m_c - M) instead of exp(x_i - M), so the argmax can differ from the
 // reference only where two scores agree to within a few fp32 roundings.  Ties go to the lowest
@@ -210,6 +211,7 @@ __global__ __launch_bounds__(kSampThreads) void sampler_chunk_kernel(
     // ---- chunk maximum of x / T (noise: the reference's division; otherwise the scale is folded
     //      into the base-2 exponent: y = x * log2(e) / T) ------------------------------------------
     const float k = 1.4426950408889634f / t_in;
+    const float inv_t = 1.0f / t_in;                       // x * (1 / T): within one ulp of the reference's x / T, a tenth of its instructions
     float m = -INFINITY;
     float xt[kNoise ? kVec : 1][8];                        // noise: x / T, kept (8 values per lane); else recomputed from `raw`
 #pragma unroll
@@ -219,7 +221,7 @@ __global__ __launch_bounds__(kSampThreads) void sampler_chunk_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             if (kNoise) {
-                xt[v][i] = x[i] / t_in;
+                xt[v][i] = x[i] * inv_t;
                 m = fmaxf(m, xt[v][i]);
             } else {
                 m = fmaxf(m, x[i] * k);
@@ -243,7 +245,7 @@ __global__ __launch_bounds__(kSampThreads) void sampler_chunk_kernel(
             for (int i = 0; i < 8; ++i) {
                 const float ex = expf(xt[v][i] - mm);      // exp(-inf) = 0 past the row end
                 ssum += ex;
-                if (c0 + i < vocab) better(best, best_i, ex / fmaxf(e[v][i], 1e-10f), c0 + i);
+                if (c0 + i < vocab) better(best, best_i, ex * __builtin_amdgcn_rcpf(fmaxf(e[v][i], 1e-10f)), c0 + i);   // (one-ulp reciprocal)
             }
         }
         ssum = wave_sum(ssum);
