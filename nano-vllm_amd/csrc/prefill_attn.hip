@@ -4,23 +4,37 @@
 // the prefix-cache case where K/V of every sequence are read through the block table.
 //
 // One workgroup of 4 wavefronts per (128-query tile, query head, sequence); wavefront w owns
-// 32 query rows.  Keys are walked in tiles of 64.  The K and V tiles ([64][128] bf16 each) are
-// double-buffered in LDS and travel global -> LDS directly (global_load_lds_dwordx4, 16 bytes per
-// lane, no vector register in between): the loads of tile t+1 are issued before the arithmetic of
-// tile t and waited for just before the one barrier per tile.  Rows keep their 256-byte pitch;
-// the 16-byte chunk index is XOR-swizzled per key (K: by key%16, V: by 4*(key%4)) -- on the
-// global side, since the LDS side of such a load is fixed -- so that the operand reads below are
-// spread over all banks.
-// Everything is computed transposed so that a query is a LANE (lane % 32) and keys / output
-// dims live in that lane's registers:
-//     S^T = K * Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q^T (registers)
-//     O^T = V^T * P^T    A = V^T through ds_read_b64_tr_b16 (LDS transpose read: 4 keys x 16
-//                        dims -> lane = dim, registers = keys), B = P^T from the S^T registers
-// The softmax state (running max, running sum) is therefore per lane, reductions over keys
-// are in-register, and the only cross-lane step is one exchange between lanes l and l^32,
-// which hold the two key halves of the same query.  The S^T accumulator layout (register i
-// of lane l = key 8*(i/4) + 4*(l/32) + i%4) is also a legal k-ordering for the B operand of
-// the second product as long as V^T uses the same key order, so P never leaves registers.
+// 32 query rows, as two groups of 16.  Keys are walked in tiles of 64.  Everything is computed
+// transposed with v_mfma_f32_16x16x32_bf16 (on this part it sustains 98 % of the matrix peak,
+// the 32x32x16 form 71-87 %), so that a query is a lane column (lane % 16) and keys / output
+// dims live in registers and across the four 16-lane groups:
+//     S^T = K * Q^T      A = 16 keys x 32 dims from LDS (one ds_read_b128), B = Q^T (registers)
+//     O^T = V^T * P^T    A = 16 dims x 32 keys through two ds_read_b64_tr_b16 (LDS transpose
+//                        read), B = P^T straight from the S^T accumulators
+// The S^T accumulator layout (register i of lane l = key 4*(l/16) + i of a 16-key block) taken
+// over two key blocks is a legal k-ordering for the B operand of the second product as long as
+// V^T is fetched in the same key order, so P never leaves registers.
+//
+// LDS.  The K and V tiles are double-buffered and travel global -> LDS directly
+// (global_load_lds_dwordx4, 16 bytes per lane, no vector register in between).  Such a load
+// writes its 64 lanes' 16-byte pieces to consecutive LDS addresses, but which piece of global
+// memory a lane fetches is free, so the LDS image is laid out fragment by fragment: one load
+// instruction fetches 64 bytes (32 dims) of 16 key rows and fills the 1 KB block that one
+// matrix operand is read from.  Within a block the four 16-byte pieces of a key are permuted
+// so that every operand read is spread over all banks, and every read address is one lane
+// constant plus an immediate offset: no address arithmetic in the loop.
+//
+// Softmax.  p = exp2(scale*log2e * s - ref), where ref follows the running maximum lazily: it is
+// raised (and the sums rescaled) only when a partial row sum shows that some p has passed
+// 2^64, which the partial sums the pass needs anyway reveal -- the common path computes no
+// maximum and exchanges nothing between lanes.  Any common factor cancels in the final
+// division by the row sum; fp32 and bf16 share their exponent range, so nothing overflows.
+// Per score that leaves one fma, one exp2, one add and half a bf16 pack.
+//
+// Schedule.  A tile is processed in two halves of 32 keys: the scores of the second half are
+// multiplied while the first half goes through the softmax, and the first half's P*V runs
+// while the second half goes through the softmax; the eight loads of the next tile are spread
+// over the four phases.  One barrier per tile.
 //
 // The causal mask is aligned to the end of the keys: query i sees keys j <= i + (Lk - Lq).
 // Work: 4 * 128 flop per (query, visible key, head).
@@ -28,21 +42,24 @@
 
 #include <math.h>
 
+#include <type_traits>
+
 namespace nva {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));   // plain vectors: stay in registers
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x8_t __attribute__((ext_vector_type(8)));
-typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
-typedef __attribute__((address_space(3))) void *lds_void_ptr;
+typedef __attribute__((address_space(3))) char *lds_char_ptr;
+typedef __attribute__((address_space(3))) u32x4_t *lds_u32x4_ptr;
+typedef __attribute__((address_space(3))) s16x4_t *lds_s16x4_ptr;
 
 constexpr int kPfThreads = 256;
 constexpr int kPfBM = 128;            // queries per workgroup
 constexpr int kPfBN = 64;             // keys per LDS tile
-constexpr int kPfTileChunks = kPfBN * 16;   // 16-byte chunks per K (or V) tile
-constexpr float kPfLazyLog2 = 8.f;    // how far (in powers of two) the running maximum may run ahead of the exponent base
+constexpr int kPfTileBytes = kPfBN * kHeadDim * 2;      // one K (or V) tile: 16 KB = 16 blocks of 1 KB
+constexpr float kPfLiftLimit = 1.2676506e30f;           // 2^100: a row sum beyond it makes the workgroup repeat its work with exact maxima
 
 struct PrefillArgs {
     const bf16_t *q; int64_t q_row_stride;
@@ -52,42 +69,30 @@ struct PrefillArgs {
     const int32_t *block_tables; int32_t bt_row_stride;
     const int32_t *cu_seqlens_q; const int32_t *cu_seqlens_k;
     bf16_t *out;
-    int32_t num_heads, num_kv_heads, num_blocks, num_q_tiles;
+    int32_t num_heads, num_kv_heads, num_blocks, num_q_tiles, batch;
     float scale_log2e;
 };
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(const u32x4_t &u) { return __builtin_bit_cast(bf16x8_t, u); }
-
-// max of three in one instruction.  (fmaxf on accumulator registers costs three: the compiler
-// first canonicalises both operands, because it cannot know that they hold no signalling NaN.)
-__device__ __forceinline__ float max3(float x, float y, float z) {
-    float r;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
-    return r;
-}
 
 // global -> LDS without a register in between: lane l's 16 bytes at base + voff land at LDS byte
 // address lds_addr + 16 l.  Written as inline assembly on purpose: the compiler would make every
 // LDS read that follows its own builtin wait for the load (it cannot tell the two LDS buffers
 // apart), which would serialise the prefetch of the next tile with the arithmetic of this one.
 // The caller waits with s_waitcnt vmcnt(0) before the barrier that publishes the tile.
-// (s_nop 3: the load needs one wait state after the write of m0, and five after a vector
-// instruction wrote one of its scalar operands -- v_readfirstlane does -- which the compiler
-// cannot provide for an instruction it does not see.)
-__device__ __forceinline__ void load_to_lds_16(const void *base, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
+// (s_nop 0: the load needs one wait state after the write of m0, which the compiler cannot provide
+// for an instruction it does not see.  Its scalar operands are always results of scalar
+// arithmetic; one written by a vector instruction -- v_readfirstlane -- would need five.)
+__device__ __forceinline__ void load_to_lds_16(const void *base, uint32_t &voff, uint32_t lds_addr) {
+    // Not volatile, and the offset register is declared as written although it keeps its value: the
+    // statement is then an ordinary instruction that the scheduler may place anywhere between the
+    // computation of its operands and the next use of the offset (a volatile statement is a fence
+    // for every LDS read and cuts the block into separately scheduled pieces).  The loads of one
+    // tensor form a chain through the offset; loads_issued() ends the chains before the wait.
+    asm("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+        : "+v"(voff) : "s"(base), "s"(lds_addr) : "m0");
 }
-
-// The same, for operands that a matrix instruction has just written.  A vector instruction may
-// read the result registers of a v_mfma_f32_32x32x16_bf16 (8 passes) no sooner than 11 cycles
-// after its issue, and the hardware does not check: the compiler pads its own instructions with
-// s_nop, but it does not look inside inline assembly, so the padding is part of the statement.
-__device__ __forceinline__ float max3_after_mfma(float x, float y, float z) {
-    float r;
-    asm volatile("s_nop 7\n\ts_nop 2\n\tv_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
-    return r;
-}
+__device__ __forceinline__ void loads_issued(uint32_t koff, uint32_t voff) { asm volatile("" :: "v"(koff), "v"(voff)); }
 
 template <bool kPaged>
 __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const PrefillArgs a) {
@@ -95,54 +100,60 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     // the kv head is the fastest index: with 8 kv heads all workgroups that read the K/V of one
     // (sequence, kv head) -- every query tile of the query heads sharing it -- run on the same XCD
     // and find those rows in its L2.  Every XCD still gets the same mix of tiles however ragged
-    // the sequences are.  Query tiles run from the last one (most keys, longest) to the first.
+    // the sequences are.  The slowest index is the query tile counted from the END of its sequence:
+    // the last tiles of all sequences (most keys, longest) are dispatched first, then the ones before
+    // them, so that the long units start early and the short ones fill the tail.
     const int group = a.num_heads / a.num_kv_heads;
     const int hkv = blockIdx.x % a.num_kv_heads;
     int rest = blockIdx.x / a.num_kv_heads;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // (in a scalar register: branches on it stay scalar)
     const int h = hkv * group + rest % group;
     rest /= group;
-    const int mt = a.num_q_tiles - 1 - rest % a.num_q_tiles;
-    const int b = rest / a.num_q_tiles;
+    const int b = rest % a.batch;
     const int q0 = a.cu_seqlens_q[b], k0 = a.cu_seqlens_k[b];
     const int lq = a.cu_seqlens_q[b + 1] - q0;
     const int lk = a.cu_seqlens_k[b + 1] - k0;
+    const int mt = (lq + kPfBM - 1) / kPfBM - 1 - rest / a.batch;
+    if (mt < 0) return;                                  // the sequence has fewer tiles; also covers empty query spans
     const int row0 = mt * kPfBM;
-    if (row0 >= lq) return;                              // also covers empty query spans
     const int off = lk - lq;                             // bottom-right causal alignment
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int qi = lane & 31, hh = lane >> 5;
-    const int qrow = row0 + wave * 32 + qi;              // query index inside the sequence
-    const bool q_valid = qrow < lq;
-    const int qrow_c = min(qrow, lq - 1);
+    const int r = lane & 15, g = lane >> 4;              // column of the 16x16 products, 16-lane group
+    const float c = a.scale_log2e;
 
-    // Q^T fragments: B operand, column = this lane's query, k = dims 16*s + 8*hh + [0,8)
-    bf16x8_t qfrag[8];
-    {
-        const bf16_t *qp = a.q + static_cast<int64_t>(q0 + qrow_c) * a.q_row_stride + h * kHeadDim + 8 * hh;
+    // Q^T fragments: B operand, column = this lane's query of group qa, k = dims 32 ks + 8 g + [0, 8)
+    int qrow[2];                                         // query index inside the sequence
+    bf16x8_t qfrag[2][4];
 #pragma unroll
-        for (int s = 0; s < 8; ++s) qfrag[s] = as_bf16x8(*reinterpret_cast<const u32x4_t *>(qp + 16 * s));
+    for (int qa = 0; qa < 2; ++qa) {
+        qrow[qa] = row0 + wave * 32 + 16 * qa + r;
+        const bf16_t *qp = a.q + static_cast<int64_t>(q0 + min(qrow[qa], lq - 1)) * a.q_row_stride + h * kHeadDim + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) qfrag[qa][ks] = as_bf16x8(*reinterpret_cast<const u32x4_t *>(qp + 32 * ks));
     }
 
-    f32x16_t oacc[4];
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
-    float m_run = -INFINITY;      // shared by lanes l and l^32
-    float l_run = 0.f;            // partial over this lane's key half
+    f32x4_t oacc[8][2];                                  // [16-dim block][query group]: dim 16 db + 4 g + i
+    // Exponent reference per query group, shared by the four lanes of a query: neg_ref = -c * (the
+    // raw score that maps to p = 1).
+    float neg_ref[2] = {0.f, 0.f};
+    // Row sums: accumulated by the matrix pipe as a product of P^T with a block of ones (every row of
+    // the 16x16 result is the sum over all 32 keys of the step), which costs 4 products per tile where
+    // 32 additions per lane would compete with the exponentials for the vector pipe.  The sums are
+    // thus taken over the bf16 values of P that the second product uses.
+    f32x4_t lacc[2];
 
-    __shared__ __attribute__((aligned(16))) u32x4_t sK[2][kPfTileChunks];
-    __shared__ __attribute__((aligned(16))) u32x4_t sV[2][kPfTileChunks];
+    // K tiles 0/1, then V tiles 0/1; a tile is 16 blocks of 1 KB, block (16-key group kb, 32-dim slice x)
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * kPfTileBytes];
+    __shared__ int retry_flag;
+    const lds_char_ptr lds = (lds_char_ptr)(&smem[0]);
 
     const int q_hi = min(row0 + kPfBM, lq) - 1;          // last query row of the tile
     const int kv_end = min(lk, q_hi + off + 1);          // keys [0, kv_end) are visible to the tile
     const int ntiles = kv_end > 0 ? (kv_end + kPfBN - 1) / kPfBN : 0;
-    const int wave_qmin = row0 + __builtin_amdgcn_readfirstlane(wave) * 32;   // (in a scalar register: branches on it stay scalar)
+    const int wave_qmin = row0 + wave * 32;
 
-    // global -> registers for key tile kt: thread t moves chunks t, t+256, t+512, t+768 of the tile
-    // (chunk c = key c/16, 16 bytes c%16); keys past the end are clamped and masked later
     // A tile of 64 keys starts at a multiple of 64 and so lies in one 256-token block: its block
     // id is the same for every lane, and it is fetched one tile ahead of the tile's own loads so
     // that no load of the loop waits for an address.
@@ -154,213 +165,321 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         // (the column is clamped to the row: cu_seqlens_k is device data the host could not check)
         return kPaged ? a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + min((kt * kPfBN) >> 8, a.bt_row_stride - 1) + lane_zero] : 0;
     };
-    // K/V tiles go from global memory straight into LDS (global_load_lds_dwordx4: every lane
-    // moves 16 bytes, the 64 lanes of one instruction fill 1 KB of LDS in lane order -- four key
-    // rows -- and no vector register or LDS store instruction is spent on staging).  The LDS side
-    // of such a load cannot be permuted, so the XOR swizzle is applied on the global side: the lane
-    // that fills slot `lane % 16` of key row `key` fetches chunk slot ^ swizzle(key) of that row.
-    // Instruction r of wavefront w covers keys 16r + 4w + [0, 4): this lane's key is tid/16 + 16r.
-    // Addressing: a tile's first row has a wave-uniform address; this lane's chunk sits a fixed
-    // 32-bit byte offset behind it, so a load needs no per-lane 64-bit arithmetic.  Only the last,
-    // partial tile clamps its rows to the last key.
-    const int lkey = tid >> 4;
-    const int lch_k = (tid & 15) ^ (lkey & 15), lch_v = (tid & 15) ^ (4 * (lkey & 3));
+
+    // ---- loads.  Wavefront w fetches key rows 16 w .. 16 w + 15 of a tile with four K and four V
+    // instructions; instruction x covers bytes 64 x .. 64 x + 63 of those rows (4 lanes per row) and
+    // fills block (w, x).  Lane 4 k + j of it fetches, for key k of the group, piece
+    //     K: j ^ (k >> 2)          V: j ^ 2 ((k >> 2) & 1)
+    // of the row's four 16-byte pieces.
+    const int lk16 = lane >> 2, lj = lane & 3;
+    const int lrow = wave * 16 + lk16;                   // this lane's key row within a tile
+    const int kpiece = lj ^ (lk16 >> 2), vpiece = lj ^ (2 * ((lk16 >> 2) & 1));
     const int64_t kstride = kPaged ? static_cast<int64_t>(a.num_kv_heads) * kHeadDim : a.k_row_stride;
     const int64_t vstride = kPaged ? kstride : a.v_row_stride;
-    const uint32_t koff0 = static_cast<uint32_t>((lkey * kstride + lch_k * 8) * 2);
-    const uint32_t voff0 = static_cast<uint32_t>((lkey * vstride + lch_v * 8) * 2);
-    const uint32_t kstep = static_cast<uint32_t>(16 * kstride * 2), vstep = static_cast<uint32_t>(16 * vstride * 2);
-    // LDS byte addresses of this wavefront's first 1 KB span in buffer 0 of each tensor
     const uint32_t lds_k0 = __builtin_amdgcn_readfirstlane(
-        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_ptr)&sK[0][wave * 64])));
-    const uint32_t lds_v0 = __builtin_amdgcn_readfirstlane(
-        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_ptr)&sV[0][wave * 64])));
-    // Issues the loads of key tile kt into LDS buffer `buf`; returns false when the tile's block
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + wave * 4096);
+    struct NextTile { const char *kb, *vb; uint32_t ko, vo, dk, dv; };
+    // Prepares the loads of key tile kt into LDS buffer `buf`; `ok` is false when the tile's block
     // table entry is out of range (the loads then read block 0 and the tile is masked out).
-    auto load_tile = [&](int kt, int32_t blk_v, int buf) __attribute__((always_inline)) {
+    auto plan_tile = [&](int kt, int32_t blk_v, int buf, bool &ok) __attribute__((always_inline)) -> NextTile {
         const int32_t blk = kPaged ? __builtin_amdgcn_readfirstlane(blk_v) : 0;
-        const bool ok = !kPaged || static_cast<uint32_t>(blk) < static_cast<uint32_t>(a.num_blocks);
+        ok = !kPaged || static_cast<uint32_t>(blk) < static_cast<uint32_t>(a.num_blocks);
         const int key0 = kt * kPfBN;
-        const char *kb, *vb;
+        NextTile t;
         if (kPaged) {
             const int64_t e = ((static_cast<int64_t>(ok ? blk : 0) * kBlockSize + (key0 & 255)) * a.num_kv_heads + hkv) *
                               kHeadDim * 2;
-            kb = reinterpret_cast<const char *>(a.k_cache) + e;
-            vb = reinterpret_cast<const char *>(a.v_cache) + e;
+            t.kb = reinterpret_cast<const char *>(a.k_cache) + e;
+            t.vb = reinterpret_cast<const char *>(a.v_cache) + e;
         } else {
-            kb = reinterpret_cast<const char *>(a.k) + (static_cast<int64_t>(k0 + key0) * kstride + hkv * kHeadDim) * 2;
-            vb = reinterpret_cast<const char *>(a.v) + (static_cast<int64_t>(k0 + key0) * vstride + hkv * kHeadDim) * 2;
+            t.kb = reinterpret_cast<const char *>(a.k) + (static_cast<int64_t>(k0 + key0) * kstride + hkv * kHeadDim) * 2;
+            t.vb = reinterpret_cast<const char *>(a.v) + (static_cast<int64_t>(k0 + key0) * vstride + hkv * kHeadDim) * 2;
         }
-        const uint32_t dk = lds_k0 + buf * (kPfTileChunks * 16), dv = lds_v0 + buf * (kPfTileChunks * 16);
-        if (key0 + kPfBN <= lk) {
+        const int row = min(lrow, lk - 1 - key0);        // rows past the last key repeat it and are masked later
+        t.ko = static_cast<uint32_t>((row * kstride + kpiece * 8) * 2);
+        t.vo = static_cast<uint32_t>((row * vstride + vpiece * 8) * 2);
+        t.dk = lds_k0 + buf * kPfTileBytes;
+        t.dv = t.dk + 2 * kPfTileBytes;
+        return t;
+    };
+    auto issue_k = [&](NextTile &t, int x) __attribute__((always_inline)) { load_to_lds_16(t.kb + 64 * x, t.ko, t.dk + 1024 * x); };
+    auto issue_v = [&](NextTile &t, int x) __attribute__((always_inline)) { load_to_lds_16(t.vb + 64 * x, t.vo, t.dv + 1024 * x); };
+
+    // ---- operand reads.  K block (kb, ks): the piece of key k holding dims 32 ks + 8 g' + [0, 8) sits at
+    // 16-byte slot 4 k + (g' ^ (k >> 2)).  V block (kb, x): key k owns 64 bytes, its two 32-byte
+    // halves (16 dims each) swapped when (k >> 2) is odd.  A transpose read of a 16-lane group covers
+    // 4 keys x 16 dims: lane r supplies the address of key r / 4, dims 4 (r % 4) .. + 3 and
+    // receives dim r of the four keys.
+    const uint32_t kread0 = 16 * (4 * r + (g ^ (r >> 2)));
+    const uint32_t vread0 = 2 * kPfTileBytes + 64 * (4 * g + (r >> 2)) + 8 * (r & 3);
+    const uint32_t vread_y0 = vread0 + 32 * (g & 1), vread_y1 = vread0 + 32 * ((g & 1) ^ 1);
+
+    const std::integral_constant<int, 0> h0;
+    const std::integral_constant<int, 1> h1;
+    f32x4_t sacc[4][2];                                  // [16-key block][query group]: key 16 kb + 4 g + i
+    u32x4_t pfrag[2][2];                                 // [32-key half][query group]
+
+    // S^T = K Q^T for the two 16-key blocks of half H
+    auto scores = [&](auto hc, lds_char_ptr kl) __attribute__((always_inline)) {
+        constexpr int H = decltype(hc)::value;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                load_to_lds_16(kb, r * kstep + koff0, dk + r * 4096);
-                load_to_lds_16(vb, r * vstep + voff0, dv + r * 4096);
+        for (int kb = 2 * H; kb < 2 * H + 2; ++kb)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const u32x4_t kf = *(lds_u32x4_ptr)(kl + (kb * 4 + ks) * 1024);
+#pragma unroll
+                for (int qa = 0; qa < 2; ++qa)
+                    sacc[kb][qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        as_bf16x8(kf), qfrag[qa][ks], ks == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : sacc[kb][qa], 0, 0, 0);
             }
-        } else {
-            const int last = lk - 1 - key0;              // >= 0: rows past it repeat it and are masked later
+    };
+    // O^T += V^T P^T over the 32 keys of half H
+    auto values = [&](auto hc, lds_char_ptr vl0, lds_char_ptr vl1) __attribute__((always_inline)) {
+        constexpr int H = decltype(hc)::value;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = min(lkey + 16 * r, last);
-                load_to_lds_16(kb, static_cast<uint32_t>((key * kstride + lch_k * 8) * 2), dk + r * 4096);
-                load_to_lds_16(vb, static_cast<uint32_t>((key * vstride + lch_v * 8) * 2), dv + r * 4096);
+        for (int db = 0; db < 8; ++db) {
+            const lds_char_ptr vl = (db & 1) ? vl1 : vl0;
+            const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(vl + ((2 * H) * 4 + (db >> 1)) * 1024));
+            const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(vl + ((2 * H + 1) * 4 + (db >> 1)) * 1024));
+            const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+            for (int qa = 0; qa < 2; ++qa)
+                oacc[db][qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both),
+                                                                       as_bf16x8(pfrag[H][qa]), oacc[db][qa], 0, 0, 0);
+        }
+    };
+    // score of register e (0..7) of half H, masked: key index kt*64 + 32 H + 16 (e/4) + 4 g + e%4
+    auto masked_score = [&](auto hc, auto dc, int qa, int e, int key_base, int limit) __attribute__((always_inline)) -> float {
+        constexpr int H = decltype(hc)::value;
+        constexpr bool kDiag = decltype(dc)::value;
+        const float s = sacc[2 * H + (e >> 2)][qa][e & 3];
+        return (kDiag && key_base + 32 * H + 16 * (e >> 2) + (e & 3) > limit) ? -INFINITY : s;
+    };
+    // running maximum of the (masked) scores of half H, per lane
+    auto row_max = [&](auto hc, int key_base, bool cur_ok, float (&m)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int qa = 0; qa < 2; ++qa) {
+            const int limit = cur_ok ? qrow[qa] + off : -1;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) m[qa] = fmaxf(m[qa], masked_score(hc, std::true_type{}, qa, e, key_base, limit));
+        }
+    };
+    // One tile of the attention proper, written out in the order it is to execute and fenced step by
+    // step (left to itself the scheduler issues every LDS read right before its use and keeps each
+    // softmax in one piece, so that reads, exponentials and products wait for one another):
+    //   1  the 8 K reads of the first half
+    //   2  its 16 products, the 8 K reads of the second half and the next tile's K loads between them
+    //   3  the second half's 16 products, each followed by one score of the first half going through
+    //      the softmax and one V read of the first half
+    //   4  the first half's 16 P V products, each followed by one score of the second half going
+    //      through the softmax and one V read of the second half
+    //   5  the second half's 16 P V products, the next tile's V loads between them
+    // A read is thus issued 8 to 16 products before its use, and the exponentials run beside products.
+    auto attend = [&](auto dc, lds_char_ptr kl, lds_char_ptr vl0, lds_char_ptr vl1, int key_base, bool cur_ok,
+                      NextTile &nxt) __attribute__((always_inline)) {
+        const int limit[2] = {cur_ok ? qrow[0] + off : -1, cur_ok ? qrow[1] + off : -1};   // last key a query may see
+        const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+        const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};     // eight bf16 1.0
+        u32x4_t kfa[8], kfb[8];
+        s16x4_t vta[16], vtb[16];
+        float pprev = 0.f;
+        // one score of half H through the softmax: j = 8 qa + e
+        auto slice = [&](auto hc, int j) __attribute__((always_inline)) {
+            constexpr int H = decltype(hc)::value;
+            const int qa = j >> 3, e = j & 7;
+            const float p = __builtin_amdgcn_exp2f(fmaf(masked_score(hc, dc, qa, e, key_base, limit[qa]), c, neg_ref[qa]));   // exp2(-inf) = 0
+            if (e & 1) pfrag[H][qa][e >> 1] = pack_bf16x2(pprev, p);
+            else pprev = p;
+        };
+        auto vread = [&](auto hc, int j) __attribute__((always_inline)) -> s16x4_t {    // j = 2 db + (0: keys 0..15, 1: keys 16..31 of the half)
+            constexpr int H = decltype(hc)::value;
+            const int db = j >> 1;
+            const lds_char_ptr vl = (db & 1) ? vl1 : vl0;
+            return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(vl + ((2 * H + (j & 1)) * 4 + (db >> 1)) * 1024));
+        };
+#pragma unroll
+        for (int i = 0; i < 8; ++i) kfa[i] = *(lds_u32x4_ptr)(kl + i * 1024);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int kb = i >> 2, ks = i & 3;
+#pragma unroll
+            for (int qa = 0; qa < 2; ++qa)
+                sacc[kb][qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kfa[i]), qfrag[qa][ks], ks == 0 ? zero : sacc[kb][qa], 0, 0, 0);
+            kfb[i] = *(lds_u32x4_ptr)(kl + (8 + i) * 1024);
+            if ((i & 1) == 0) issue_k(nxt, i >> 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int i = j >> 1, qa = j & 1, kb = 2 + (i >> 2), ks = i & 3;
+            sacc[kb][qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kfb[i]), qfrag[qa][ks], ks == 0 ? zero : sacc[kb][qa], 0, 0, 0);
+            slice(h0, j);
+            vta[j] = vread(h0, j);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int qa = 0; qa < 2; ++qa)
+            lacc[qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(pfrag[0][qa]), lacc[qa], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int db = j >> 1, qa = j & 1;
+            const s16x8_t both = __builtin_shufflevector(vta[2 * db], vta[2 * db + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+            oacc[db][qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), as_bf16x8(pfrag[0][qa]), oacc[db][qa], 0, 0, 0);
+            slice(h1, j);
+            vtb[j] = vread(h1, j);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int qa = 0; qa < 2; ++qa)
+            lacc[qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(pfrag[1][qa]), lacc[qa], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int db = j >> 1, qa = j & 1;
+            const s16x8_t both = __builtin_shufflevector(vtb[2 * db], vtb[2 * db + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+            oacc[db][qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), as_bf16x8(pfrag[1][qa]), oacc[db][qa], 0, 0, 0);
+            if ((j & 3) == 0) issue_v(nxt, j >> 2);
+            if (j & 1) __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    int retry_pending = 0;
+
+    // One pass over the key tiles.  kExact = false: the attention itself, with the exponent reference
+    // taken from the first 32 keys.  kExact = true: only the scores, for the exact row maxima.
+    auto pass = [&](auto xc) __attribute__((always_inline)) {
+        constexpr bool kExact = decltype(xc)::value;
+        float m_exact[2] = {-INFINITY, -INFINITY};
+        bool tile_ok = true;                             // of the tile computed next
+        int32_t blk_next = 0;                            // block id of the tile loaded next
+        if (ntiles > 0) {
+            NextTile t = plan_tile(0, fetch_block(0), 0, tile_ok);
+#pragma unroll
+            for (int x = 0; x < 4; ++x) { issue_k(t, x); issue_v(t, x); }
+            loads_issued(t.ko, t.vo);
+        }
+        if (ntiles > 1) blk_next = fetch_block(1);
+        // Everything loaded so far (Q above all) is waited for here, and the Q fragments are then
+        // passed through an empty asm.  Without this the compiler keeps treating them as in flight
+        // inside the loop and makes each product wait for the loads issued just before it -- the
+        // next tile's prefetch -- which put a full memory round trip into every tile.
+        __builtin_amdgcn_s_waitcnt(0x0F70);              // vmcnt(0): also the first tile has landed in LDS
+#pragma unroll
+        for (int qa = 0; qa < 2; ++qa)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) asm volatile("" : "+v"(qfrag[qa][ks]));
+        __syncthreads();
+
+        if (!kExact) {
+#pragma unroll
+            for (int db = 0; db < 8; ++db)
+#pragma unroll
+                for (int qa = 0; qa < 2; ++qa) oacc[db][qa] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            lacc[0] = lacc[1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            if (retry_pending == 0 && ntiles > 0) {
+                // exponent reference: the largest score among the first 32 keys of the row.  Whatever it
+                // is cancels in the final division; it only has to keep every p inside fp32 range.
+                float m[2] = {-INFINITY, -INFINITY};
+                scores(h0, lds + kread0);
+                row_max(h0, 4 * g, tile_ok, m);
+#pragma unroll
+                for (int qa = 0; qa < 2; ++qa) {
+                    m[qa] = fmaxf(m[qa], __shfl_xor(m[qa], 16, 64));
+                    m[qa] = fmaxf(m[qa], __shfl_xor(m[qa], 32, 64));
+                    neg_ref[qa] = m[qa] == -INFINITY ? 0.f : -m[qa] * c;
+                }
             }
         }
-        return ok;
+
+        // Per wavefront the tiles come in three runs: those wholly below the diagonal for all of its 32
+        // queries (no mask), those that cross it, and those wholly beyond it, of which only the loads
+        // are this wavefront's business (they exist because later wavefronts of the workgroup see
+        // them).  One loop per run, so that each loop has a single body.
+        const int n_active = min(ntiles, (wave_qmin + 31 + off) / kPfBN + 1);                 // wave_qmin + 31 + off >= 0 or no tile at all
+        const int n_plain = wave_qmin + off + 1 >= kPfBN ? min(n_active, (wave_qmin + off + 1) / kPfBN) : 0;
+        auto step = [&](int kt, auto dc, auto cc) __attribute__((always_inline)) {
+            constexpr bool kCompute = decltype(cc)::value;
+            const int buf = kt & 1;
+            const bool cur_ok = tile_ok;
+            // the next tile lands in the other buffer during this tile's arithmetic (that buffer was last
+            // read before the previous barrier); after the last tile the same tile is fetched once more
+            // rather than giving the loop a second body without loads
+            NextTile nxt = plan_tile(min(kt + 1, ntiles - 1), blk_next, buf ^ 1, tile_ok);
+            if (kt + 2 < ntiles) blk_next = fetch_block(kt + 2);
+            if (kCompute) {
+                const lds_char_ptr kl = lds + (kread0 + buf * kPfTileBytes);
+                const lds_char_ptr vl0 = lds + (vread_y0 + buf * kPfTileBytes), vl1 = lds + (vread_y1 + buf * kPfTileBytes);
+                const int key_base = kt * kPfBN + 4 * g; // key of register 0 of block 0
+                if (kExact) {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) issue_k(nxt, x);
+                    scores(h0, kl);
+                    scores(h1, kl);
+                    row_max(h0, key_base, cur_ok, m_exact);
+                    row_max(h1, key_base, cur_ok, m_exact);
+                } else {
+                    attend(dc, kl, vl0, vl1, key_base, cur_ok, nxt);
+                }
+            } else {
+#pragma unroll
+                for (int x = 0; x < 4; ++x) { issue_k(nxt, x); if (!kExact) issue_v(nxt, x); }
+            }
+            loads_issued(nxt.ko, nxt.vo);
+            __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wavefront's part of the next tile is in LDS
+            __syncthreads();
+        };
+        int kt = 0;
+        for (; kt < n_plain; ++kt) {
+            if (kPaged && !tile_ok) step(kt, std::true_type{}, std::false_type{});  // (a tile behind a bad block id is masked out: nothing to add)
+            else step(kt, std::false_type{}, std::true_type{});
+        }
+        for (; kt < n_active; ++kt) step(kt, std::true_type{}, std::true_type{});
+        for (; kt < ntiles; ++kt) step(kt, std::true_type{}, std::false_type{});
+        if (kExact) {
+#pragma unroll
+            for (int qa = 0; qa < 2; ++qa) {
+                m_exact[qa] = fmaxf(m_exact[qa], __shfl_xor(m_exact[qa], 16, 64));
+                m_exact[qa] = fmaxf(m_exact[qa], __shfl_xor(m_exact[qa], 32, 64));
+                neg_ref[qa] = m_exact[qa] == -INFINITY ? 0.f : -m_exact[qa] * c;
+            }
+        }
     };
 
-    bool tile_ok = true;                                 // of the tile computed next
-    int32_t blk_next = 0;                                // block id of the tile loaded next
-    if (ntiles > 0) tile_ok = load_tile(0, fetch_block(0), 0);
-    if (ntiles > 1) blk_next = fetch_block(1);
-    // Everything loaded so far (Q above all) is waited for here, and the Q fragments are then
-    // passed through an empty asm.  Without this the compiler keeps treating them as in flight
-    // inside the loop and makes each product wait for the loads issued just before it -- the
-    // next tile's prefetch -- which put a full memory round trip into every tile.
-    __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0): also the first tile has landed in LDS
+    // First with the cheap reference.  If a row sum of the workgroup then lies beyond 2^100 (or is not a
+    // number), some score exceeded the first 32 keys' maximum by hundreds: the workgroup computes the
+    // exact row maxima in a pass of their own and repeats the attention with them (p <= 1).
+    float l_tot[2];
+    for (;;) {
+        pass(std::false_type{});
+        bool beyond = false;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) asm volatile("" : "+v"(qfrag[s]));
-    __syncthreads();
-
-    for (int kt = 0; kt < ntiles; ++kt) {
-        const int buf = kt & 1;
-        const bool more = kt + 1 < ntiles;
-        const bool cur_ok = tile_ok;
-        if (more) {                                      // lands in the other buffer during this tile's arithmetic
-            tile_ok = load_tile(kt + 1, blk_next, buf ^ 1);   // (that buffer was last read before the previous barrier)
-            if (kt + 2 < ntiles) blk_next = fetch_block(kt + 2);
+        for (int qa = 0; qa < 2; ++qa) {
+            l_tot[qa] = lacc[qa][0];
+            beyond |= !(l_tot[qa] <= kPfLiftLimit);
         }
-
-        // A wavefront skips the arithmetic of a tile that lies wholly beyond the diagonal for all
-        // of its 32 queries (the tile exists because later wavefronts of the workgroup see it).
-        if (kt * kPfBN <= wave_qmin + 31 + off) {
-        // ---- S^T = K Q^T for two 32-key sub-tiles ----------------------------------------
-        f32x16_t sacc[2];
-        // (the two wavefronts that share a SIMD belong to different workgroups; the one in a matrix
-        // phase is given priority over the one in its softmax phase, so that the matrix pipe is fed
-        // first: measured 3 % faster)
-        __builtin_amdgcn_s_setprio(2);
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) sacc[t2][i] = 0.f;
-#pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const int key = t2 * 32 + qi;
-                const u32x4_t kf = sK[buf][key * 16 + ((2 * s + hh) ^ (key & 15))];
-                sacc[t2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf), qfrag[s], sacc[t2], 0, 0, 0);
-            }
-        }
-
-        __builtin_amdgcn_s_setprio(0);
-        // ---- causal mask, running softmax (base 2; the scale is folded into the exponent) -------
-        const int limit = cur_ok ? qrow + off : -1;      // last key this query may see
-        if ((kt * kPfBN + kPfBN - 1) > (wave_qmin + off) || !cur_ok) {   // only tiles that cross the diagonal
-            const int key_base = kt * kPfBN + 4 * hh;
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    if (key_base + t2 * 32 + 8 * (i >> 2) + (i & 3) > limit) sacc[t2][i] = -INFINITY;
-        }
-        // one dependent chain per sub-tile, so that every read of an accumulator follows the padded first one
-        float mloc0 = max3_after_mfma(sacc[0][0], sacc[0][1], sacc[0][2]);
-        float mloc1 = max3_after_mfma(sacc[1][0], sacc[1][1], sacc[1][2]);
-#pragma unroll
-        for (int i = 3; i < 15; i += 2) {
-            mloc0 = max3(mloc0, sacc[0][i], sacc[0][i + 1]);
-            mloc1 = max3(mloc1, sacc[1][i], sacc[1][i + 1]);
-        }
-        mloc1 = max3(mloc1, sacc[1][15], sacc[0][15]);   // (behind both padded reads)
-        const float mloc = max3(mloc0, mloc1, mloc1);
-        // m_run is the reference point of the exponentials, p = exp2(scale*log2e * (s - m_run)).  It
-        // follows the true running maximum lazily: only when the maximum has moved more than
-        // kPfLazyLog2 powers of two past it are the sums rescaled (p stays below 2^kPfLazyLog2, far
-        // inside fp32 / bf16 range, and the final division by the row sum cancels the common
-        // factor exactly).  With an eager update nearly every tile of a short sequence moves the
-        // maximum of some query of the wavefront, and every move costs 64 multiplications per lane.
-        const float m_true = max3(m_run, mloc, __shfl_xor(mloc, 32, 64));
-        const bool lift = (m_true - m_run) * a.scale_log2e > kPfLazyLog2;   // -inf - -inf = NaN: false
-        if (__builtin_amdgcn_ballot_w64(lift) != 0) {
-            const float m_to = lift ? m_true : m_run;
-            const float alpha = lift ? __builtin_amdgcn_exp2f((m_run - m_to) * a.scale_log2e) : 1.f;   // 0 on first use
-            l_run *= alpha;
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-            m_run = m_to;
-        }
-        const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;    // no key seen yet: p = 0
-        const float neg_ms = -m_safe * a.scale_log2e;
-        float ps[4] = {0.f, 0.f, 0.f, 0.f};              // four short chains instead of one of 32 adds
-        u32x4_t pfrag[2][2];                             // [sub-tile][k-step of 16 keys]
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-            float p[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                p[i] = __builtin_amdgcn_exp2f(fmaf(sacc[t2][i], a.scale_log2e, neg_ms));   // exp2(-inf) = 0
-                ps[i & 3] += p[i];
-            }
-#pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2)
-                pfrag[t2][s2] = u32x4_t{pack_bf16x2(p[8 * s2 + 0], p[8 * s2 + 1]), pack_bf16x2(p[8 * s2 + 2], p[8 * s2 + 3]),
-                                        pack_bf16x2(p[8 * s2 + 4], p[8 * s2 + 5]), pack_bf16x2(p[8 * s2 + 6], p[8 * s2 + 7])};
-        }
-        l_run += (ps[0] + ps[1]) + (ps[2] + ps[3]);
-
-        // ---- O^T += V^T P^T ----------------------------------------------------------------
-        // A operand: row = output dim (dt*32 + lane%32), k slot (hh, i) = key 16*s2 + 8*(i/4) + 4*hh + i%4.
-        // Transpose read: the 16 lanes of a group fetch [4 keys][16 dims]; lane r16 supplies the address
-        // of key r16/4, dims 4*(r16%4)..+3 and receives dim r16 of the four keys.
-        {
-            __builtin_amdgcn_s_setprio(2);
-            const int r16 = lane & 15;
-            const int dsub = (lane >> 4) & 1;            // which 16-dim half of the 32-dim tile
-            const int kq = r16 >> 2;                     // key within the group of four
-            const int cin = dsub * 2 + ((r16 >> 1) & 1); // 16-byte chunk within the tile's 64-byte dim span
-            const char *vbase = reinterpret_cast<const char *>(&sV[buf][0]) + (r16 & 1) * 8;
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-                    for (int s2 = 0; s2 < 2; ++s2) {
-                        const int k_lo = t2 * 32 + 16 * s2 + 4 * hh + kq;     // k slots 0..3
-                        const int k_hi = k_lo + 8;                            // k slots 4..7
-                        const int c = dt * 4 + cin;
-                        const s16x4_t vlo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (lds_s16x4_ptr)(vbase + k_lo * 256 + ((c ^ (4 * (k_lo & 3))) * 16)));
-                        const s16x4_t vhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (lds_s16x4_ptr)(vbase + k_hi * 256 + ((c ^ (4 * (k_hi & 3))) * 16)));
-                        const s16x8_t both = __builtin_shufflevector(vlo, vhi, 0, 1, 2, 3, 4, 5, 6, 7);
-                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, both),
-                                                                           as_bf16x8(pfrag[t2][s2]), oacc[dt], 0, 0, 0);
-                    }
-            __builtin_amdgcn_s_setprio(0);
-        }
-
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70);              // vmcnt(0): this wavefront's part of the next tile is in LDS
+        if (retry_pending) break;
+        if (tid == 0) retry_flag = 0;
         __syncthreads();
+        if (beyond) retry_flag = 1;
+        __syncthreads();
+        if (retry_flag == 0) break;
+        retry_pending = 1;
+        pass(std::true_type{});
     }
 
-    // ---- normalise and store: register i of tile dt = dim dt*32 + 8*(i/4) + 4*hh + i%4 ----
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    if (q_valid) {
-        bf16_t *op = a.out + (static_cast<int64_t>(q0 + qrow) * a.num_heads + h) * kHeadDim + 4 * hh;
+    // ---- normalise and store: register i of block db = dim 16 db + 4 g + i ----
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+    for (int qa = 0; qa < 2; ++qa) {
+        const float inv = l_tot[qa] > 0.f ? 1.f / l_tot[qa] : 0.f;
+        if (qrow[qa] < lq) {
+            bf16_t *op = a.out + (static_cast<int64_t>(q0 + qrow[qa]) * a.num_heads + h) * kHeadDim + 4 * g;
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
+            for (int db = 0; db < 8; ++db) {
                 uint2 w;
-                w.x = pack_bf16x2(oacc[dt][4 * g4 + 0] * inv, oacc[dt][4 * g4 + 1] * inv);
-                w.y = pack_bf16x2(oacc[dt][4 * g4 + 2] * inv, oacc[dt][4 * g4 + 3] * inv);
-                *reinterpret_cast<uint2 *>(op + dt * 32 + 8 * g4) = w;
+                w.x = pack_bf16x2(oacc[db][qa][0] * inv, oacc[db][qa][1] * inv);
+                w.y = pack_bf16x2(oacc[db][qa][2] * inv, oacc[db][qa][3] * inv);
+                *reinterpret_cast<uint2 *>(op + 16 * db) = w;
             }
+        }
     }
 }
 
@@ -412,6 +531,7 @@ extern "C" int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride, cons
     a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.num_blocks = num_blocks;
     a.scale_log2e = scale * 1.4426950408889634f;
     a.num_q_tiles = (max_seqlen_q + kPfBM - 1) / kPfBM;
+    a.batch = batch;
     if (static_cast<int64_t>(a.num_q_tiles) * num_heads * batch > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;
     const dim3 grid(static_cast<uint32_t>(a.num_q_tiles) * num_heads * batch);
     hipStream_t s = static_cast<hipStream_t>(stream);
