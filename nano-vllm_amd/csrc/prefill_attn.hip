@@ -275,8 +275,9 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     //      through the softmax and one V read of the second half
     //   5  the second half's 16 P V products, the next tile's V loads between them
     // A read is thus issued 8 to 16 products before its use, and the exponentials run beside products.
-    auto attend = [&](auto dc, lds_char_ptr kl, lds_char_ptr vl0, lds_char_ptr vl1, int key_base, bool cur_ok,
+    auto attend = [&](auto dc, auto lc, lds_char_ptr kl, lds_char_ptr vl0, lds_char_ptr vl1, int key_base, bool cur_ok,
                       NextTile &nxt) __attribute__((always_inline)) {
+        constexpr bool kLoads = decltype(lc)::value;       // false for the last tile of the pass: nothing follows it
         const int limit[2] = {cur_ok ? qrow[0] + off : -1, cur_ok ? qrow[1] + off : -1};   // last key a query may see
         const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
         const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};     // eight bf16 1.0
@@ -307,7 +308,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
             for (int qa = 0; qa < 2; ++qa)
                 sacc[kb][qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kfa[i]), qfrag[qa][ks], ks == 0 ? zero : sacc[kb][qa], 0, 0, 0);
             kfb[i] = *(lds_u32x4_ptr)(kl + (8 + i) * 1024);
-            if ((i & 1) == 0) issue_k(nxt, i >> 1);
+            if (kLoads && (i & 1) == 0) issue_k(nxt, i >> 1);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -338,7 +339,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
             const int db = j >> 1, qa = j & 1;
             const s16x8_t both = __builtin_shufflevector(vtb[2 * db], vtb[2 * db + 1], 0, 1, 2, 3, 4, 5, 6, 7);
             oacc[db][qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), as_bf16x8(pfrag[1][qa]), oacc[db][qa], 0, 0, 0);
-            if ((j & 3) == 0) issue_v(nxt, j >> 2);
+            if (kLoads && (j & 3) == 0) issue_v(nxt, j >> 2);
             if (j & 1) __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -396,44 +397,56 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         // them).  One loop per run, so that each loop has a single body.
         const int n_active = min(ntiles, (wave_qmin + 31 + off) / kPfBN + 1);                 // wave_qmin + 31 + off >= 0 or no tile at all
         const int n_plain = wave_qmin + off + 1 >= kPfBN ? min(n_active, (wave_qmin + off + 1) / kPfBN) : 0;
-        auto step = [&](int kt, auto dc, auto cc) __attribute__((always_inline)) {
+        // lc = false: the last tile of the pass.  Nothing is loaded during it and nobody waits after it.
+        auto step = [&](int kt, auto dc, auto cc, auto lc) __attribute__((always_inline)) {
             constexpr bool kCompute = decltype(cc)::value;
+            constexpr bool kLoads = decltype(lc)::value;
             const int buf = kt & 1;
             const bool cur_ok = tile_ok;
             // the next tile lands in the other buffer during this tile's arithmetic (that buffer was last
-            // read before the previous barrier); after the last tile the same tile is fetched once more
-            // rather than giving the loop a second body without loads
-            NextTile nxt = plan_tile(min(kt + 1, ntiles - 1), blk_next, buf ^ 1, tile_ok);
-            if (kt + 2 < ntiles) blk_next = fetch_block(kt + 2);
+            // read before the previous barrier)
+            NextTile nxt = {};
+            if (kLoads) {
+                nxt = plan_tile(kt + 1, blk_next, buf ^ 1, tile_ok);
+                if (kt + 2 < ntiles) blk_next = fetch_block(kt + 2);
+            }
             if (kCompute) {
                 const lds_char_ptr kl = lds + (kread0 + buf * kPfTileBytes);
                 const lds_char_ptr vl0 = lds + (vread_y0 + buf * kPfTileBytes), vl1 = lds + (vread_y1 + buf * kPfTileBytes);
                 const int key_base = kt * kPfBN + 4 * g; // key of register 0 of block 0
                 if (kExact) {
+                    if (kLoads) {
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) issue_k(nxt, x);
+                        for (int x = 0; x < 4; ++x) issue_k(nxt, x);
+                    }
                     scores(h0, kl);
                     scores(h1, kl);
                     row_max(h0, key_base, cur_ok, m_exact);
                     row_max(h1, key_base, cur_ok, m_exact);
                 } else {
-                    attend(dc, kl, vl0, vl1, key_base, cur_ok, nxt);
+                    attend(dc, lc, kl, vl0, vl1, key_base, cur_ok, nxt);
                 }
-            } else {
+            } else if (kLoads) {
 #pragma unroll
                 for (int x = 0; x < 4; ++x) { issue_k(nxt, x); if (!kExact) issue_v(nxt, x); }
             }
-            loads_issued(nxt.ko, nxt.vo);
-            __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wavefront's part of the next tile is in LDS
-            __syncthreads();
+            if (kLoads) {
+                loads_issued(nxt.ko, nxt.vo);
+                __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): this wavefront's part of the next tile is in LDS
+                __syncthreads();
+            }
         };
+        const std::true_type yes;
+        const std::false_type no;
+        const int last = ntiles - 1;
         int kt = 0;
-        for (; kt < n_plain; ++kt) {
-            if (kPaged && !tile_ok) step(kt, std::true_type{}, std::false_type{});  // (a tile behind a bad block id is masked out: nothing to add)
-            else step(kt, std::false_type{}, std::true_type{});
+        for (; kt < min(n_plain, last); ++kt) {
+            if (kPaged && !tile_ok) step(kt, yes, no, yes);     // (a tile behind a bad block id is masked out: nothing to add)
+            else step(kt, no, yes, yes);
         }
-        for (; kt < n_active; ++kt) step(kt, std::true_type{}, std::true_type{});
-        for (; kt < ntiles; ++kt) step(kt, std::true_type{}, std::false_type{});
+        for (; kt < min(n_active, last); ++kt) step(kt, yes, yes, yes);
+        for (; kt < last; ++kt) step(kt, yes, no, yes);
+        if (last >= 0 && last < n_active) step(last, yes, yes, no);    // (with the mask, needed or not: one body fewer)
         if (kExact) {
 #pragma unroll
             for (int qa = 0; qa < 2; ++qa) {

@@ -190,3 +190,55 @@ def test_prefill_one_sequence_dominates(dev, hq, hkv, q_lens):
                                   num_blocks=40)
     out, want = _paged(case, dev)
     assert_attn_close(out, want, "dominant sequence, paged")
+
+
+@pytest.mark.parametrize("boost_from,factor", [(32, 40.0), (200, 60.0), (0, 50.0)])
+def test_prefill_scores_far_beyond_the_first_keys(dev, boost_from, factor):
+    """The kernel takes its exponent reference from the first 32 keys of a row and repeats a query
+    tile with exact row maxima when a row sum shows that this was not enough.  Keys from
+    `boost_from` on are scaled so that their scores exceed the first keys' by many hundreds (raw
+    score standard deviation ~ 11 * factor), which overflows every p computed against the cheap
+    reference; with boost_from = 0 the large scores are in the first keys instead and everything
+    after them underflows.  Packed and through the block table; rows see between 1 and ~900 keys."""
+    q_lens, prefix = [300, 129, 64, 500], [1, 0, 2, 0]
+    case = synthetic.prefill_case(seed=31, q_lens=q_lens, prefix_blocks=[0] * 4, num_blocks=40)
+    k = case.k.clone()
+    for s in range(len(q_lens)):
+        a, b = int(case.cu_seqlens_q[s]), int(case.cu_seqlens_q[s + 1])
+        if boost_from == 0:
+            k[a:min(a + 20, b)] = (k[a:min(a + 20, b)].float() * factor).to(torch.bfloat16)
+        elif a + boost_from < b:
+            k[a + boost_from:b] = (k[a + boost_from:b].float() * factor).to(torch.bfloat16)
+    packed = synthetic.PrefillCase(case.q, k, case.v, case.k_cache, case.v_cache, case.cu_seqlens_q, case.cu_seqlens_k,
+                                   case.max_seqlen_q, case.max_seqlen_k, case.slot_mapping, None, case.scale)
+    out, want = _packed(packed, dev)
+    assert_attn_close(out, want, f"boosted keys from {boost_from}, packed")
+    paged = synthetic.prefill_case(seed=32, q_lens=q_lens, prefix_blocks=prefix, num_blocks=40)
+    k2 = paged.k.clone()
+    for s in range(len(q_lens)):
+        a, b = int(paged.cu_seqlens_q[s]), int(paged.cu_seqlens_q[s + 1])
+        lo = a if boost_from == 0 else min(a + boost_from, b)
+        hi = min(a + 20, b) if boost_from == 0 else b
+        k2[lo:hi] = (k2[lo:hi].float() * factor).to(torch.bfloat16)
+    paged = synthetic.PrefillCase(paged.q, k2, paged.v, paged.k_cache, paged.v_cache, paged.cu_seqlens_q,
+                                  paged.cu_seqlens_k, paged.max_seqlen_q, paged.max_seqlen_k, paged.slot_mapping,
+                                  paged.block_tables, paged.scale)
+    out, want = _paged(paged, dev)
+    assert_attn_close(out, want, f"boosted keys from {boost_from}, paged")
+
+
+def test_prefill_rows_without_any_key_are_zero(dev):
+    """More queries than keys (cu_seqlens_k shorter than cu_seqlens_q): with the mask aligned to the end
+    of the keys the first Lq - Lk queries see nothing and come out as zeros, as the oracle's do."""
+    g = torch.Generator().manual_seed(41)
+    lq, lk = 200, 70
+    q = torch.randn((lq, 4, 128), generator=g).to(torch.bfloat16)
+    k = torch.randn((lk, 2, 128), generator=g).to(torch.bfloat16)
+    v = torch.randn((lk, 2, 128), generator=g).to(torch.bfloat16)
+    cu_q, cu_k = torch.tensor([0, lq], dtype=torch.int32), torch.tensor([0, lk], dtype=torch.int32)
+    out = varlen_prefill_attention(q.to(dev), k.to(dev), v.to(dev), cu_q.to(dev), cu_k.to(dev), lq, lk, 128 ** -0.5)
+    torch.cuda.synchronize()
+    want = oracle.varlen_prefill_attention(q, k, v, cu_q, cu_k, 128 ** -0.5, precision="fp32")
+    assert float(want[:lq - lk].abs().max()) == 0.0
+    assert float(out[:lq - lk].float().abs().max()) == 0.0
+    assert_attn_close(out, want, "more queries than keys")
