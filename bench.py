@@ -157,28 +157,57 @@ def bench_prefill(args, dev):
     import torch
     import nanovllm_amd as nva
     from nanovllm_amd import synthetic
-    c = synthetic.prefill_case(seed=0)
-    q, k, v, kc, vc = (t.to(dev) for t in (c.q, c.k, c.v, c.k_cache, c.v_cache))
-    cq, ck, sm, bt = (t.to(dev) for t in (c.cu_seqlens_q, c.cu_seqlens_k, c.slot_mapping, c.block_tables))
-    nva.store_kvcache(k, v, kc, vc, sm)
-    fn = lambda: nva.varlen_prefill_attention(q, kc, vc, cq, ck, c.max_seqlen_q, c.max_seqlen_k, c.scale,
-                                              block_table=bt)
+    uniform = getattr(args, "uniform", None)
+    if uniform:
+        # S packed sequences of L tokens each, no prefix cache: the matrix-bound end of the prefill kernel
+        n_seq, seq_len = (int(x) for x in uniform.lower().split("x"))
+        hq, hkv, d = 16, 8, 128
+        g = torch.Generator(device=dev).manual_seed(3)
+        q = torch.randn(n_seq * seq_len, hq, d, device=dev, generator=g).to(torch.bfloat16)
+        k = torch.randn(n_seq * seq_len, hkv, d, device=dev, generator=g).to(torch.bfloat16)
+        v = torch.randn(n_seq * seq_len, hkv, d, device=dev, generator=g).to(torch.bfloat16)
+        cu = torch.arange(0, (n_seq + 1) * seq_len, seq_len, dtype=torch.int32, device=dev)
+        fn = lambda: nva.varlen_prefill_attention(q, k, v, cu, cu, seq_len, seq_len, d ** -0.5)
+        flops = n_seq * 4 * d * hq * (seq_len * (seq_len + 1) // 2)
+        what = "varlen_prefill_attn: %d packed sequences of %d tokens, no prefix cache, 16q/8kv heads, head_dim 128" % (n_seq, seq_len)
+        metric = "causal varlen prefill attention, achieved TFLOP/s (%d x %d tokens)" % (n_seq, seq_len)
+        kernel, total_q, c = "prefill_attn_kernel<packed>", n_seq * seq_len, None
+    else:
+        c = synthetic.prefill_case(seed=0)
+        q, k, v, kc, vc = (t.to(dev) for t in (c.q, c.k, c.v, c.k_cache, c.v_cache))
+        cq, ck, sm, bt = (t.to(dev) for t in (c.cu_seqlens_q, c.cu_seqlens_k, c.slot_mapping, c.block_tables))
+        nva.store_kvcache(k, v, kc, vc, sm)
+        fn = lambda: nva.varlen_prefill_attention(q, kc, vc, cq, ck, c.max_seqlen_q, c.max_seqlen_k, c.scale,
+                                                  block_table=bt)
+        flops = c.algorithmic_flops
+        what = ("varlen_prefill_attn config3: 16 sequences, Lq U[100,1024], half with 1-3 cached "
+                "256-token prefix blocks, 16q/8kv heads, head_dim 128")
+        metric = "causal varlen prefill attention with prefix cache, achieved TFLOP/s (config 3)"
+        kernel, total_q = "prefill_attn_kernel<paged>", int(c.q.shape[0])
     ms = _event_time_ms([fn], args.steps, args.warmup)
     per_step_ms = ms / args.steps
-    flops = c.algorithmic_flops
     tflops = flops / (per_step_ms * 1e-3) / 1e12
     result = {
-        "metric": "causal varlen prefill attention with prefix cache, achieved TFLOP/s (config 3)",
+        "metric": metric,
         "value": round(tflops, 2), "unit": "TFLOP/s", "ms_per_step": round(per_step_ms, 5),
-        "config": {"workload": "varlen_prefill_attn config3: 16 sequences, Lq U[100,1024], half with 1-3 cached "
-                               "256-token prefix blocks, 16q/8kv heads, head_dim 128", "total_q": int(c.q.shape[0])},
+        "config": {"workload": what, "total_q": total_q},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "prefill_attn_kernel<paged>", "algorithmic_flops_per_launch": int(flops)},
+                     "kernel": kernel, "algorithmic_flops_per_launch": int(flops)},
     }
 
     def cpu():
         import oracle
+        if c is None:
+            # one sequence cut to 2048 tokens: the full size would take the host minutes
+            n = min(2048, q.shape[0])
+            qc, kc_, vc_ = q[:n].cpu(), k[:n].cpu(), v[:n].cpu()
+            one = torch.tensor([0, n], dtype=torch.int32)
+            sec = _median_cpu_seconds(lambda: oracle.varlen_prefill_attention(qc, kc_, vc_, one, one, 128 ** -0.5, precision="sdpa"), repeats=3)
+            fl = 4 * 128 * 16 * (n * (n + 1) // 2)
+            return {"value": round(fl / sec / 1e12, 4), "unit": "TFLOP/s", **_cpu_cores(), "kind": "port",
+                    "sample": "one sequence of %d tokens, bf16 torch SDPA with explicit lower-right mask, median of 3" % n,
+                    "seconds": round(sec, 3)}
         ek, ev = c.k_cache.clone(), c.v_cache.clone()
         oracle.store_kvcache(c.k, c.v, ek, ev, c.slot_mapping)
         sec = _median_cpu_seconds(lambda: oracle.varlen_prefill_attention(
@@ -436,6 +465,7 @@ def collect_extra(dev, model, prompts, params):
     extra = {}
     for name, fn, steps, kw in (("scatter_config1", bench_scatter, 400, {}), ("rope_scatter_16384_tokens", bench_rope_scatter, 100, {}),
                                 ("decode_config2", bench_decode, 112, {}), ("prefill_config3", bench_prefill, 50, {}),
+                                ("prefill_2x16384_tokens", bench_prefill, 10, {"uniform": "2x16384"}),
                                 ("sampler_256x151936", bench_sampler, 100, {}),
                                 ("sampler_with_noise_256x151936", bench_sampler, 50, {"noise": True}),
                                 ("decode_config5_shape", bench_decode_longctx_shape, 1, {})):
@@ -610,6 +640,7 @@ def main():
     ap.add_argument("--tokens", type=int, default=None, help="scatter / rope-scatter: number of tokens (default 4096 / 16384)")
     ap.add_argument("--contiguous", action="store_true", help="scatter: slots in ascending order instead of a random permutation")
     ap.add_argument("--noise", action="store_true", help="sampler: time the replayable path that reads an Exp(1) noise tensor")
+    ap.add_argument("--uniform", default=None, metavar="SxL", help="prefill: S packed sequences of L tokens each instead of config 3 (e.g. 2x16384)")
     ap.add_argument("--bucket-step", type=int, default=16, help="e2e only: spacing of the captured decode batch sizes")
     ap.add_argument("--no-extra", action="store_true", help="e2e only: skip the per-configuration rooflines and the eager pass")
     args = ap.parse_args()

@@ -69,7 +69,7 @@ struct PrefillArgs {
     const int32_t *block_tables; int32_t bt_row_stride;
     const int32_t *cu_seqlens_q; const int32_t *cu_seqlens_k;
     bf16_t *out;
-    int32_t num_heads, num_kv_heads, num_blocks, num_q_tiles, batch;
+    int32_t num_heads, num_kv_heads, num_blocks, num_q_tiles;
     float scale_log2e;
 };
 
@@ -100,9 +100,10 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     // the kv head is the fastest index: with 8 kv heads all workgroups that read the K/V of one
     // (sequence, kv head) -- every query tile of the query heads sharing it -- run on the same XCD
     // and find those rows in its L2.  Every XCD still gets the same mix of tiles however ragged
-    // the sequences are.  The slowest index is the query tile counted from the END of its sequence:
-    // the last tiles of all sequences (most keys, longest) are dispatched first, then the ones before
-    // them, so that the long units start early and the short ones fill the tail.
+    // the sequences are.  Query tiles run from the last one (most keys, longest) to the first, sequence
+    // by sequence: the tiles of one sequence run close together in time and share its K/V in L2
+    // (handing out the last tiles of ALL sequences first, then the ones before them, takes as long
+    // and fetches twice as much from memory: 7 MB of K/V per kv head do not stay in a 4 MB L2).
     const int group = a.num_heads / a.num_kv_heads;
     const int hkv = blockIdx.x % a.num_kv_heads;
     int rest = blockIdx.x / a.num_kv_heads;
@@ -111,13 +112,13 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // (in a scalar register: branches on it stay scalar)
     const int h = hkv * group + rest % group;
     rest /= group;
-    const int b = rest % a.batch;
+    const int mt = a.num_q_tiles - 1 - rest % a.num_q_tiles;
+    const int b = rest / a.num_q_tiles;
     const int q0 = a.cu_seqlens_q[b], k0 = a.cu_seqlens_k[b];
     const int lq = a.cu_seqlens_q[b + 1] - q0;
     const int lk = a.cu_seqlens_k[b + 1] - k0;
-    const int mt = (lq + kPfBM - 1) / kPfBM - 1 - rest / a.batch;
-    if (mt < 0) return;                                  // the sequence has fewer tiles; also covers empty query spans
     const int row0 = mt * kPfBM;
+    if (row0 >= lq) return;                              // also covers empty query spans
     const int off = lk - lq;                             // bottom-right causal alignment
 
     const int r = lane & 15, g = lane >> 4;              // column of the 16x16 products, 16-lane group
@@ -169,11 +170,11 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     // ---- loads.  Wavefront w fetches key rows 16 w .. 16 w + 15 of a tile with four K and four V
     // instructions; instruction x covers bytes 64 x .. 64 x + 63 of those rows (4 lanes per row) and
     // fills block (w, x).  Lane 4 k + j of it fetches, for key k of the group, piece
-    //     K: j ^ (k >> 2)          V: j ^ 2 ((k >> 2) & 1)
+    //     K: j ^ (-(k >> 2) & 3)   V: j ^ 2 ((k >> 2) & 1)
     // of the row's four 16-byte pieces.
     const int lk16 = lane >> 2, lj = lane & 3;
     const int lrow = wave * 16 + lk16;                   // this lane's key row within a tile
-    const int kpiece = lj ^ (lk16 >> 2), vpiece = lj ^ (2 * ((lk16 >> 2) & 1));
+    const int kpiece = lj ^ ((0 - (lk16 >> 2)) & 3), vpiece = lj ^ (2 * ((lk16 >> 2) & 1));
     const int64_t kstride = kPaged ? static_cast<int64_t>(a.num_kv_heads) * kHeadDim : a.k_row_stride;
     const int64_t vstride = kPaged ? kstride : a.v_row_stride;
     const uint32_t lds_k0 = __builtin_amdgcn_readfirstlane(
@@ -206,11 +207,18 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     auto issue_v = [&](NextTile &t, int x) __attribute__((always_inline)) { load_to_lds_16(t.vb + 64 * x, t.vo, t.dv + 1024 * x); };
 
     // ---- operand reads.  K block (kb, ks): the piece of key k holding dims 32 ks + 8 g' + [0, 8) sits at
-    // 16-byte slot 4 k + (g' ^ (k >> 2)).  V block (kb, x): key k owns 64 bytes, its two 32-byte
+    // 16-byte slot 4 k + (g' ^ (-(k >> 2) & 3)).  V block (kb, x): key k owns 64 bytes, its two 32-byte
     // halves (16 dims each) swapped when (k >> 2) is odd.  A transpose read of a 16-lane group covers
     // 4 keys x 16 dims: lane r supplies the address of key r / 4, dims 4 (r % 4) .. + 3 and
     // receives dim r of the four keys.
-    const uint32_t kread0 = 16 * (4 * r + (g ^ (r >> 2)));
+    // Which lanes have to fall into different banks was measured: a 64-bit read serves lanes 0-31 in one
+    // LDS cycle and 32-63 in the next; a 128-bit read serves 16 lanes per cycle, and they are not 16
+    // neighbours but four aligned groups of four lanes: of the eight such groups of each half of the
+    // wavefront, the ones numbered 0, 3, 5, 6 in one cycle and 1, 2, 4, 7 in the other.  The K
+    // permutation above puts the four groups of a cycle on the four residues of the slot number
+    // modulo 4 (with k >> 2 in place of -(k >> 2) & 3 groups 0 and 5 collide and every K read takes
+    // twice as long).
+    const uint32_t kread0 = 16 * (4 * r + (g ^ ((0 - (r >> 2)) & 3)));
     const uint32_t vread0 = 2 * kPfTileBytes + 64 * (4 * g + (r >> 2)) + 8 * (r & 3);
     const uint32_t vread_y0 = vread0 + 32 * (g & 1), vread_y1 = vread0 + 32 * ((g & 1) ^ 1);
 
@@ -544,7 +552,6 @@ extern "C" int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride, cons
     a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.num_blocks = num_blocks;
     a.scale_log2e = scale * 1.4426950408889634f;
     a.num_q_tiles = (max_seqlen_q + kPfBM - 1) / kPfBM;
-    a.batch = batch;
     if (static_cast<int64_t>(a.num_q_tiles) * num_heads * batch > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;
     const dim3 grid(static_cast<uint32_t>(a.num_q_tiles) * num_heads * batch);
     hipStream_t s = static_cast<hipStream_t>(stream);
