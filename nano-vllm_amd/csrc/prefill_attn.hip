@@ -485,6 +485,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         if (retry_flag == 0) break;
         retry_pending = 1;
         pass(std::true_type{});
+        __syncthreads();                                 // (its last tile is still being read while a faster wavefront would already load tile 0 again)
     }
 
     // ---- normalise and store: register i of block db = dim 16 db + 4 g + i ----
