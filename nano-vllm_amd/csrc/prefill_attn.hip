@@ -477,7 +477,10 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
             l_tot[qa] = lacc[qa][0];
             beyond |= !(l_tot[qa] <= kPfLiftLimit);
         }
-        if (retry_pending) break;
+        if (retry_pending) {
+            __syncthreads();                             // (the output tiles go through the LDS the last tile is read from)
+            break;
+        }
         if (tid == 0) retry_flag = 0;
         __syncthreads();
         if (beyond) retry_flag = 1;
@@ -488,20 +491,31 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         __syncthreads();                                 // (its last tile is still being read while a faster wavefront would already load tile 0 again)
     }
 
-    // ---- normalise and store: register i of block db = dim 16 db + 4 g + i ----
+    // ---- normalise and store.  Register i of block db is dim 16 db + 4 g + i of one query: stored from
+    // there a lane would write 8 bytes here and 8 bytes 32 bytes further on.  Each wavefront passes its
+    // 32 x 128 tile through LDS instead (the K/V tiles are done with; rows 272 bytes apart, so that the
+    // 64-bit writes of 32 lanes fall into 32 different bank pairs) and stores whole rows, 16 bytes per lane.
+    constexpr int kOutPitch = 2 * kHeadDim + 16;
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(3))) u32x2_t *lds_u32x2_ptr;
+    const lds_char_ptr ow = lds + wave * (32 * kOutPitch);
 #pragma unroll
     for (int qa = 0; qa < 2; ++qa) {
         const float inv = l_tot[qa] > 0.f ? 1.f / l_tot[qa] : 0.f;
-        if (qrow[qa] < lq) {
-            bf16_t *op = a.out + (static_cast<int64_t>(q0 + qrow[qa]) * a.num_heads + h) * kHeadDim + 4 * g;
 #pragma unroll
-            for (int db = 0; db < 8; ++db) {
-                uint2 w;
-                w.x = pack_bf16x2(oacc[db][qa][0] * inv, oacc[db][qa][1] * inv);
-                w.y = pack_bf16x2(oacc[db][qa][2] * inv, oacc[db][qa][3] * inv);
-                *reinterpret_cast<uint2 *>(op + 16 * db) = w;
-            }
+        for (int db = 0; db < 8; ++db) {
+            const u32x2_t w = {pack_bf16x2(oacc[db][qa][0] * inv, oacc[db][qa][1] * inv),
+                               pack_bf16x2(oacc[db][qa][2] * inv, oacc[db][qa][3] * inv)};
+            *(lds_u32x2_ptr)(ow + (16 * qa + r) * kOutPitch + (16 * db + 4 * g) * 2) = w;
         }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int orow = 4 * i + (lane >> 4);
+        const u32x4_t w = *(lds_u32x4_ptr)(ow + orow * kOutPitch + (lane & 15) * 16);
+        const int qr = row0 + wave * 32 + orow;
+        if (qr < lq)
+            *reinterpret_cast<u32x4_t *>(a.out + (static_cast<int64_t>(q0 + qr) * a.num_heads + h) * kHeadDim + (lane & 15) * 8) = w;
     }
 }
 
