@@ -114,6 +114,21 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     rest /= group;
     const int mt = a.num_q_tiles - 1 - rest % a.num_q_tiles;
     const int b = rest / a.num_q_tiles;
+    // A tile of 64 keys starts at a multiple of 64 and so lies in one 256-token block: its block
+    // id is the same for every lane, and it is fetched one tile ahead of the tile's own loads so
+    // that no load of the loop waits for an address.
+    // (The id is kept in a vector register until it is used: were the compiler to see that it is
+    // uniform it would move it to a scalar register at once, and wait for every load issued before.)
+    int lane_zero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
+    auto fetch_block = [&](int kt) __attribute__((always_inline)) -> int32_t {
+        // (the column is clamped to the row: cu_seqlens_k is device data the host could not check)
+        return kPaged ? a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + min((kt * kPfBN) >> 8, a.bt_row_stride - 1) + lane_zero] : 0;
+    };
+    // (the ids of the first tiles depend on the sequence only: asked for together with its bounds, one trip
+    // to memory instead of two in a row)
+    const int32_t blk_first = fetch_block(0), blk_second = fetch_block(1);
+
     const int q0 = a.cu_seqlens_q[b], k0 = a.cu_seqlens_k[b];
     const int lq = a.cu_seqlens_q[b + 1] - q0;
     const int lk = a.cu_seqlens_k[b + 1] - k0;
@@ -154,18 +169,6 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     const int kv_end = min(lk, q_hi + off + 1);          // keys [0, kv_end) are visible to the tile
     const int ntiles = kv_end > 0 ? (kv_end + kPfBN - 1) / kPfBN : 0;
     const int wave_qmin = row0 + wave * 32;
-
-    // A tile of 64 keys starts at a multiple of 64 and so lies in one 256-token block: its block
-    // id is the same for every lane, and it is fetched one tile ahead of the tile's own loads so
-    // that no load of the loop waits for an address.
-    // (The id is kept in a vector register until it is used: were the compiler to see that it is
-    // uniform it would move it to a scalar register at once, and wait for every load issued before.)
-    int lane_zero;
-    asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
-    auto fetch_block = [&](int kt) __attribute__((always_inline)) -> int32_t {
-        // (the column is clamped to the row: cu_seqlens_k is device data the host could not check)
-        return kPaged ? a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + min((kt * kPfBN) >> 8, a.bt_row_stride - 1) + lane_zero] : 0;
-    };
 
     // ---- loads.  Wavefront w fetches key rows 16 w .. 16 w + 15 of a tile with four K and four V
     // instructions; instruction x covers bytes 64 x .. 64 x + 63 of those rows (4 lanes per row) and
@@ -361,12 +364,12 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         bool tile_ok = true;                             // of the tile computed next
         int32_t blk_next = 0;                            // block id of the tile loaded next
         if (ntiles > 0) {
-            NextTile t = plan_tile(0, fetch_block(0), 0, tile_ok);
+            NextTile t = plan_tile(0, blk_first, 0, tile_ok);
 #pragma unroll
             for (int x = 0; x < 4; ++x) { issue_k(t, x); issue_v(t, x); }
             loads_issued(t.ko, t.vo);
         }
-        if (ntiles > 1) blk_next = fetch_block(1);
+        if (ntiles > 1) blk_next = blk_second;
         // Everything loaded so far (Q above all) is waited for here, and the Q fragments are then
         // passed through an empty asm.  Without this the compiler keeps treating them as in flight
         // inside the loop and makes each product wait for the loads issued just before it -- the
