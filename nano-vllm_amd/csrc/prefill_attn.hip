@@ -387,7 +387,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
 #pragma unroll
                 for (int qa = 0; qa < 2; ++qa) oacc[db][qa] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             lacc[0] = lacc[1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            if (retry_pending == 0 && ntiles > 0) {
+            if (retry_pending == 0 && ntiles > 0 && wave_qmin < lq) {
                 // exponent reference: the largest score among the first 32 keys of the row.  Whatever it
                 // is cancels in the final division; it only has to keep every p inside fp32 range.
                 float m[2] = {-INFINITY, -INFINITY};
@@ -406,7 +406,8 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         // queries (no mask), those that cross it, and those wholly beyond it, of which only the loads
         // are this wavefront's business (they exist because later wavefronts of the workgroup see
         // them).  One loop per run, so that each loop has a single body.
-        const int n_active = min(ntiles, (wave_qmin + 31 + off) / kPfBN + 1);                 // wave_qmin + 31 + off >= 0 or no tile at all
+        // (a wavefront whose 32 rows all lie past the end of the sequence only helps with the loads)
+        const int n_active = wave_qmin >= lq ? 0 : min(ntiles, (wave_qmin + 31 + off) / kPfBN + 1);   // wave_qmin + 31 + off >= 0 or no tile at all
         const int n_plain = wave_qmin + off + 1 >= kPfBN ? min(n_active, (wave_qmin + off + 1) / kPfBN) : 0;
         // lc = false: the last tile of the pass.  Nothing is loaded during it and nobody waits after it.
         auto step = [&](int kt, auto dc, auto cc, auto lc) __attribute__((always_inline)) {
