@@ -244,21 +244,6 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
                         as_bf16x8(kf), qfrag[qa][ks], ks == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : sacc[kb][qa], 0, 0, 0);
             }
     };
-    // O^T += V^T P^T over the 32 keys of half H
-    auto values = [&](auto hc, lds_char_ptr vl0, lds_char_ptr vl1) __attribute__((always_inline)) {
-        constexpr int H = decltype(hc)::value;
-#pragma unroll
-        for (int db = 0; db < 8; ++db) {
-            const lds_char_ptr vl = (db & 1) ? vl1 : vl0;
-            const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(vl + ((2 * H) * 4 + (db >> 1)) * 1024));
-            const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(vl + ((2 * H + 1) * 4 + (db >> 1)) * 1024));
-            const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-            for (int qa = 0; qa < 2; ++qa)
-                oacc[db][qa] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both),
-                                                                       as_bf16x8(pfrag[H][qa]), oacc[db][qa], 0, 0, 0);
-        }
-    };
     // score of register e (0..7) of half H, masked: key index kt*64 + 32 H + 16 (e/4) + 4 g + e%4
     auto masked_score = [&](auto hc, auto dc, int qa, int e, int key_base, int limit) __attribute__((always_inline)) -> float {
         constexpr int H = decltype(hc)::value;
