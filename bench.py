@@ -12,6 +12,7 @@ already resident in HBM.  Workloads (shapes are the five benchmark configuration
     prefill   causal varlen prefill, 16 sequences, half with cached prefix        (config 3)
     sampler   temperature sampling over 256 x 151,936 logits (--noise: the replayable path with an Exp(1) tensor)
     rope-scatter  q/k norm + rotary + cache write in one kernel, 16,384 tokens (the scatter the engine runs)
+    glue      residual add + RMSNorm (--glue add-rms-norm) or SiLU(gate) * up (--glue silu-mul), 16,384 rows (--tokens N)
     decode-e2e-shape / decode-longctx-shape / copy   profiling helpers: the decode attention of configs 4 / 5
               alone (one layer); a plain copy of known size
 The line carries `roofline` (algorithmic bytes or flops of the dominant kernel per launch,
@@ -260,6 +261,40 @@ def bench_sampler(args, dev):
                 "kind": "port", "sample": "64 of the 256 rows, eager torch sampler with pre-drawn noise, "
                                           "median of 5", "seconds": round(sec, 4)}
     return result, cpu
+
+
+def bench_glue(args, dev):
+    """The elementwise steps either side of the attention, as the engine runs them between its GEMMs:
+    residual add + RMSNorm and SiLU(gate) * up, Qwen3-0.6B widths, a prefill-sized batch of rows."""
+    import torch
+    from nanovllm_amd.engine import layers
+    n, hidden, inter = (getattr(args, "tokens", None) or 16384), 1024, 3072
+    which = getattr(args, "glue", None) or "add-rms-norm"
+    g = torch.Generator(device=dev).manual_seed(2)
+    fns = []
+    if which == "add-rms-norm":
+        w = torch.ones(hidden, dtype=torch.bfloat16, device=dev)
+        for _ in range(3):
+            x = torch.randn(n, hidden, device=dev, generator=g).to(torch.bfloat16)
+            r = torch.randn(n, hidden, device=dev, generator=g).to(torch.bfloat16)
+            fns.append(lambda x=x, r=r: layers.add_rms_norm(x, r, w, 1e-6))
+        alg = n * hidden * 2 * 4 + hidden * 2            # x and the residual in, both results out
+        kernel = "rms_norm_kernel<2, true>"
+    else:
+        for _ in range(3):
+            x = torch.randn(n, 2 * inter, device=dev, generator=g).to(torch.bfloat16)
+            fns.append(lambda x=x: layers.silu_and_mul(x))
+        alg = n * inter * 2 * 3                          # gate and up in, the product out
+        kernel = "silu_and_mul_kernel"
+    ms = _event_time_ms(fns, args.steps, args.warmup) / args.steps
+    gbps = alg / (ms * 1e-3) / 1e9
+    result = {"metric": "%s, achieved HBM GB/s" % which, "value": round(gbps, 1), "unit": "GB/s", "ms_per_step": round(ms, 5),
+              "config": {"workload": "%s: %d rows, hidden 1024 / intermediate 3072 (Qwen3-0.6B), output allocated per call as in the engine" % (which, n),
+                         "tokens": n},
+              "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": kernel,
+                           "algorithmic_bytes_per_launch": alg}}
+    return result, (lambda: None)
 
 
 def bench_rope_scatter(args, dev):
@@ -622,9 +657,9 @@ def bench_longctx(args, dev):
     return result, (lambda: None)
 
 
-WORKLOADS = {"rope-scatter": bench_rope_scatter, "e2e": bench_e2e, "longctx": bench_longctx, "decode-e2e-shape": bench_decode_e2e_shape,
+WORKLOADS = {"rope-scatter": bench_rope_scatter, "glue": bench_glue, "e2e": bench_e2e, "longctx": bench_longctx, "decode-e2e-shape": bench_decode_e2e_shape,
              "decode-longctx-shape": bench_decode_longctx_shape, "copy": bench_copy, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
-DEFAULT_STEPS = {"rope-scatter": 100, "e2e": 1, "longctx": 1, "decode-e2e-shape": 1, "decode-longctx-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
+DEFAULT_STEPS = {"rope-scatter": 100, "glue": 100, "e2e": 1, "longctx": 1, "decode-e2e-shape": 1, "decode-longctx-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
 
 
 def main():
@@ -640,6 +675,7 @@ def main():
     ap.add_argument("--tokens", type=int, default=None, help="scatter / rope-scatter: number of tokens (default 4096 / 16384)")
     ap.add_argument("--contiguous", action="store_true", help="scatter: slots in ascending order instead of a random permutation")
     ap.add_argument("--noise", action="store_true", help="sampler: time the replayable path that reads an Exp(1) noise tensor")
+    ap.add_argument("--glue", choices=["add-rms-norm", "silu-mul"], default="add-rms-norm", help="glue: which elementwise kernel")
     ap.add_argument("--uniform", default=None, metavar="SxL", help="prefill: S packed sequences of L tokens each instead of config 3 (e.g. 2x16384)")
     ap.add_argument("--bucket-step", type=int, default=16, help="e2e only: spacing of the captured decode batch sizes")
     ap.add_argument("--no-extra", action="store_true", help="e2e only: skip the per-configuration rooflines and the eager pass")

@@ -188,7 +188,10 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const bf16_t *__restr
     unpack8(*reinterpret_cast<const uint4 *>(xr + inter + e), u);
     float y[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) y[i] = round_bf16(g[i] / (1.0f + expf(-g[i]))) * u[i];
+    // (silu through the hardware exp2 and reciprocal, one ulp each: the library expf and an IEEE division are
+    // ~25 instructions per element and made this kernel instruction-bound at prefill sizes)
+    for (int i = 0; i < 8; ++i)
+        y[i] = round_bf16(g[i] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g[i]))) * u[i];
     uint4 o;
     o.x = pack_bf16x2(y[0], y[1]); o.y = pack_bf16x2(y[2], y[3]);
     o.z = pack_bf16x2(y[4], y[5]); o.w = pack_bf16x2(y[6], y[7]);
