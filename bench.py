@@ -22,6 +22,8 @@ divided by its average duration measured with HIP events on the launch stream) a
 configurations and of the long-context decode shape, each timed in isolation in the same run, and
 one eager (no hipGraph) pass of the same workload.  Every timed e2e pass generates from prompts
 the engine has not seen (fresh draw per pass), like the reference's bench.py:22-27.
+The scatter workload is timed as one replayed hipGraph of its K launches (a Python call costs as much
+as that 7 us kernel; the eager-loop figure is reported beside it).
 Only one GPU is used; --gpus above 1 is refused.
 """
 import argparse
