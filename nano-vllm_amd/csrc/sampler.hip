@@ -224,10 +224,11 @@ __global__ __launch_bounds__(kSampThreads) void sampler_chunk_kernel(
                 xt[v][i] = x[i] * inv_t;
                 m = fmaxf(m, xt[v][i]);
             } else {
-                m = fmaxf(m, x[i] * k);
+                m = fmaxf(m, x[i]);                        // scaled once below: k > 0, so max(x) * k == max(x * k) bit for bit
             }
         }
     }
+    if (!kNoise) m *= k;
     m = wave_max(m);
     if (lane == 0) sh_max[wave] = m;
     __syncthreads();
