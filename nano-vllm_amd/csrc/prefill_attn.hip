@@ -24,17 +24,20 @@
 // so that every operand read is spread over all banks, and every read address is one lane
 // constant plus an immediate offset: no address arithmetic in the loop.
 //
-// Softmax.  p = exp2(scale*log2e * s - ref), where ref follows the running maximum lazily: it is
-// raised (and the sums rescaled) only when a partial row sum shows that some p has passed
-// 2^64, which the partial sums the pass needs anyway reveal -- the common path computes no
-// maximum and exchanges nothing between lanes.  Any common factor cancels in the final
-// division by the row sum; fp32 and bf16 share their exponent range, so nothing overflows.
-// Per score that leaves one fma, one exp2, one add and half a bf16 pack.
+// Softmax.  p = exp2(scale*log2e * s - ref) with ONE exponent reference per query for the whole
+// pass: the largest score among the first 32 keys of the row.  Any reference cancels in the final
+// division by the row sum; it only has to keep every p inside fp32 range (which bf16 shares).  The
+// common path therefore computes no maximum, rescales nothing and exchanges nothing between lanes.
+// If a row sum of the workgroup ends beyond 2^100 or is not a number, some score exceeded the
+// first keys' maximum by hundreds: the workgroup then computes the exact row maxima in a pass of
+// their own (scores only) and repeats its query tile with them.  Row sums are accumulated on the
+// matrix pipe (P^T times a block of ones), over the bf16 values of P that the second product uses.
+// Per score that leaves one fma, one exp2 and half a bf16 pack on the vector pipe.
 //
-// Schedule.  A tile is processed in two halves of 32 keys: the scores of the second half are
-// multiplied while the first half goes through the softmax, and the first half's P*V runs
-// while the second half goes through the softmax; the eight loads of the next tile are spread
-// over the four phases.  One barrier per tile.
+// Schedule.  A tile is processed in two halves of 32 keys, written out in execution order and
+// fenced step by step: the scores of the second half are multiplied while the first half goes
+// through the softmax, and the first half's P*V runs while the second half goes through the
+// softmax; the eight loads of the next tile are spread over the products.  One barrier per tile.
 //
 // The causal mask is aligned to the end of the keys: query i sees keys j <= i + (Lk - Lq).
 // Work: 4 * 128 flop per (query, visible key, head).
