@@ -9,7 +9,7 @@
  * launch; a non-zero return means nothing was enqueued.
  *
  * Dtypes / geometry: bf16 tensors, int32 index tensors, head_dim 128, KV block size 256,
- * num_heads / num_kv_heads in {1, 2, 4, 8}.  Anything else is rejected with
+ * num_heads / num_kv_heads from 1 to 8.  Anything else is rejected with
  * NVA_ERR_UNSUPPORTED_GEOMETRY rather than served by a slow path.
  *
  * File:line citations name the reference (nano-vllm) interface each entry point replaces.

@@ -555,7 +555,7 @@ extern "C" int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride
     if (head_dim != kHeadDim || block_size != kBlockSize) return NVA_ERR_UNSUPPORTED_GEOMETRY;
     if (num_heads % num_kv_heads != 0) return NVA_ERR_UNSUPPORTED_GEOMETRY;
     const int group = num_heads / num_kv_heads;
-    if (group != 1 && group != 2 && group != 4 && group != 8) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+    if (group > 8) return NVA_ERR_UNSUPPORTED_GEOMETRY;                       // (every group from 1 to 8 is built)
     if (batch == 0) return NVA_OK;
     if (static_cast<int64_t>(max_blocks) * kStagesPerBlock * num_kv_heads * kDecMaxBatch > 0x7fffffffLL)
         return NVA_ERR_BAD_SHAPE;                                             // stage counts are int32
@@ -599,7 +599,11 @@ extern "C" int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride
         switch (group) {
             case 1: rc = launch_decode<1>(a, reuse, s); break;
             case 2: rc = launch_decode<2>(a, reuse, s); break;
+            case 3: rc = launch_decode<3>(a, reuse, s); break;
             case 4: rc = launch_decode<4>(a, reuse, s); break;
+            case 5: rc = launch_decode<5>(a, reuse, s); break;
+            case 6: rc = launch_decode<6>(a, reuse, s); break;
+            case 7: rc = launch_decode<7>(a, reuse, s); break;
             default: rc = launch_decode<8>(a, reuse, s); break;
         }
         if (rc != NVA_OK) return rc;

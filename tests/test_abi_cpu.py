@@ -84,7 +84,7 @@ def test_decode_validation_and_workspace_size():
     assert call(bt=None) == _lib.ERR_NULL_POINTER
     assert call(dh=64) == _lib.ERR_UNSUPPORTED_GEOMETRY
     assert call(bs=128) == _lib.ERR_UNSUPPORTED_GEOMETRY
-    assert call(hq=24, hkv=8) == _lib.ERR_UNSUPPORTED_GEOMETRY        # group 3
+    assert call(hq=72, hkv=8) == _lib.ERR_UNSUPPORTED_GEOMETRY        # group 9 (1 to 8 are built)
     assert call(hq=16, hkv=3) == _lib.ERR_UNSUPPORTED_GEOMETRY
     assert call(qs=1024) == _lib.ERR_BAD_STRIDE
     assert call(bts=4) == _lib.ERR_BAD_STRIDE
