@@ -8,7 +8,7 @@ extern "C" const char *nva_status_string(int status) {
         case NVA_OK: return "ok";
         case NVA_ERR_NULL_POINTER: return "null pointer";
         case NVA_ERR_BAD_SHAPE: return "bad shape";
-        case NVA_ERR_UNSUPPORTED_GEOMETRY: return "unsupported geometry (head_dim 128, block_size 256, GQA group 1 to 8 only)";
+        case NVA_ERR_UNSUPPORTED_GEOMETRY: return "unsupported geometry (head_dim 128, block_size 256 * 2^k up to 4096, GQA group 1 to 8 only)";
         case NVA_ERR_BAD_STRIDE: return "bad stride";
         case NVA_ERR_MISALIGNED: return "pointer not 16-byte aligned";
         case NVA_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";

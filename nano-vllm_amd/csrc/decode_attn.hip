@@ -3,7 +3,7 @@
 // Replaces flash_attn_with_kvcache as called by nanovllm/layers/attention.py:71-74.
 //
 // Work decomposition.  The unit of work is a "stage": 32 consecutive tokens of one kv head of
-// one sequence (8 KB of K + 8 KB of V; a stage never straddles a 256-token KV block).  All
+// one sequence (8 KB of K + 8 KB of V; a stage never straddles a KV block: blocks hold 256 * 2^k tokens).  All
 // stages of the batch form one list ordered by (sequence, kv head, position) -- its length N
 // follows from context_lens alone, which every workgroup prefix-sums in LDS.  The launch is
 // a fixed set of W = 2048 wavefront "workers" (512 workgroups x 4) and worker w takes the
@@ -62,7 +62,6 @@ constexpr int kDecGrid = 512;                       // workgroups; 2 per CU on a
 constexpr int kDecWorkers = kDecGrid * kDecWaves;   // wavefront workers
 constexpr int kDecMaxBatch = 1024;                  // sequences per launch (prefix sums live in LDS)
 constexpr int kStageTok = 32;                       // tokens per stage
-constexpr int kStagesPerBlock = kBlockSize / kStageTok;
 constexpr int kStageLoads = kStageTok / 4;          // dwordx4 loads per lane per stage and tensor
 constexpr int kWaveLdsChunks = 2 * kStageTok * 16;  // K then V, in 16-byte chunks
 
@@ -86,6 +85,7 @@ struct DecodeArgs {
     float *part_ml;          // [rows][2]
     float *part_o;           // [rows][128]
     int32_t batch, max_blocks, num_heads, num_kv_heads, num_blocks;
+    int32_t block_shift;     // log2 of the tokens per KV block (256, 512, ... : a power of two)
     float scale_log2e;
 };
 
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
     // Block and number of valid rows (minus one) of stage ss of sequence bb.
     auto locate = [&](int bb, int ss, int32_t &blk, int &last) __attribute__((always_inline)) {
         last = min(kStageTok, sh_ctx[bb] - ss * kStageTok) - 1;                // in [0, 31]
-        blk = a.block_tables[static_cast<int64_t>(bb) * a.bt_row_stride + ss / kStagesPerBlock];
+        blk = a.block_tables[static_cast<int64_t>(bb) * a.bt_row_stride + (ss >> (a.block_shift - 5))];
         if (static_cast<uint32_t>(blk) >= static_cast<uint32_t>(a.num_blocks)) {
             blk = 0;                                  // bad table entry: contributes nothing
             last = -1;
@@ -123,8 +123,8 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
     // rows are clamped to the last valid row of the stage, so only rows that were written are touched.
     auto issue = [&](int bb, int gg, int ss, int32_t blk, int last, u32x4_t (&kr)[kStageLoads],
                      u32x4_t (&vr)[kStageLoads], u32x4_t (&qr)[4]) __attribute__((always_inline)) {
-        const int tok0 = (ss % kStagesPerBlock) * kStageTok;
-        const int64_t base = (static_cast<int64_t>(blk) * kBlockSize + tok0) * row + gg * kHeadDim + r16 * 8;
+        const int tok0 = (ss << 5) & ((1 << a.block_shift) - 1);       // (kStageTok = 32 tokens per stage)
+        const int64_t base = ((static_cast<int64_t>(blk) << a.block_shift) + tok0) * row + gg * kHeadDim + r16 * 8;
         const bf16_t *kb = a.k_cache + base;
         const bf16_t *vb = a.v_cache + base;
         const int lastc = max(last, 0);
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
                 int c = 0;
                 if (bi < a.batch) {
                     // a context that does not fit the table is clipped to it instead of read out of bounds
-                    const int ctx = min(max(a.context_lens[bi], 0), a.max_blocks * kBlockSize);
+                    const int ctx = min(max(a.context_lens[bi], 0), a.max_blocks << a.block_shift);
                     sh_ctx[bi] = ctx;
                     c = (ctx + kStageTok - 1) / kStageTok * hkv;
                 }
@@ -552,12 +552,13 @@ extern "C" int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride
     if (plan != NVA_PLAN_BUILD && plan != NVA_PLAN_REUSE) return NVA_ERR_BAD_SHAPE;
     if (batch < 0 || num_heads <= 0 || num_kv_heads <= 0 || max_blocks < 0 || num_blocks < 0)
         return NVA_ERR_BAD_SHAPE;
-    if (head_dim != kHeadDim || block_size != kBlockSize) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+    const int block_shift = block_shift_of(block_size);
+    if (head_dim != kHeadDim || block_shift < 0) return NVA_ERR_UNSUPPORTED_GEOMETRY;
     if (num_heads % num_kv_heads != 0) return NVA_ERR_UNSUPPORTED_GEOMETRY;
     const int group = num_heads / num_kv_heads;
     if (group > 8) return NVA_ERR_UNSUPPORTED_GEOMETRY;                       // (every group from 1 to 8 is built)
     if (batch == 0) return NVA_OK;
-    if (static_cast<int64_t>(max_blocks) * kStagesPerBlock * num_kv_heads * kDecMaxBatch > 0x7fffffffLL)
+    if (static_cast<int64_t>(max_blocks) * (block_size / kStageTok) * num_kv_heads * kDecMaxBatch > 0x7fffffffLL)
         return NVA_ERR_BAD_SHAPE;                                             // stage counts are int32
     if (!q || !k_cache || !v_cache || !context_lens || !out || !workspace) return NVA_ERR_NULL_POINTER;
     if (max_blocks > 0 && !block_tables) return NVA_ERR_NULL_POINTER;
@@ -587,6 +588,7 @@ extern "C" int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride
     a.num_heads = num_heads;
     a.num_kv_heads = num_kv_heads;
     a.num_blocks = num_blocks;
+    a.block_shift = block_shift;
     a.scale_log2e = scale * 1.4426950408889634f;
     // launches of at most kDecMaxBatch sequences each, back to back on the stream
     for (int32_t b0 = 0; b0 < batch; b0 += kDecMaxBatch) {

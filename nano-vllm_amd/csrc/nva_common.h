@@ -9,7 +9,7 @@
 namespace nva {
 
 constexpr int kHeadDim = 128;    // the only head_dim the kernels are built for
-constexpr int kBlockSize = 256;  // tokens per KV block (nanovllm/config.py:17,22)
+constexpr int kBlockSize = 256;  // smallest KV block, in tokens (nanovllm/config.py:17,22: multiples of 256)
 constexpr int kWave = 64;        // CDNA wavefront width
 
 using bf16_t = uint16_t;         // raw bf16 bits
@@ -69,6 +69,13 @@ __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, __shfl_xor(v, 16, 64));
     v = fmaxf(v, __shfl_xor(v, 32, 64));
     return v;
+}
+
+// log2 of a KV block size the kernels are built for (256, 512, 1024, 2048, 4096 tokens), else -1
+inline int block_shift_of(int32_t block_size) {
+    for (int sh = 8; sh <= 12; ++sh)
+        if (block_size == (1 << sh)) return sh;
+    return -1;
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -73,6 +73,7 @@ struct PrefillArgs {
     const int32_t *cu_seqlens_q; const int32_t *cu_seqlens_k;
     bf16_t *out;
     int32_t num_heads, num_kv_heads, num_blocks, num_q_tiles;
+    int32_t block_shift;     // log2 of the tokens per KV block
     float scale_log2e;
 };
 
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     rest /= group;
     const int mt = a.num_q_tiles - 1 - rest % a.num_q_tiles;
     const int b = rest / a.num_q_tiles;
-    // A tile of 64 keys starts at a multiple of 64 and so lies in one 256-token block: its block
+    // A tile of 64 keys starts at a multiple of 64 and so lies in one KV block (256 * 2^k tokens): its block
     // id is the same for every lane, and it is fetched one tile ahead of the tile's own loads so
     // that no load of the loop waits for an address.
     // (The id is kept in a vector register until it is used: were the compiler to see that it is
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
     asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
     auto fetch_block = [&](int kt) __attribute__((always_inline)) -> int32_t {
         // (the column is clamped to the row: cu_seqlens_k is device data the host could not check)
-        return kPaged ? a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + min((kt * kPfBN) >> 8, a.bt_row_stride - 1) + lane_zero] : 0;
+        return kPaged ? a.block_tables[static_cast<int64_t>(b) * a.bt_row_stride + min((kt * kPfBN) >> a.block_shift, a.bt_row_stride - 1) + lane_zero] : 0;
     };
     // (the ids of the first tiles depend on the sequence only: asked for together with its bounds, one trip
     // to memory instead of two in a row)
@@ -194,7 +195,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
         const int key0 = kt * kPfBN;
         NextTile t;
         if (kPaged) {
-            const int64_t e = ((static_cast<int64_t>(ok ? blk : 0) * kBlockSize + (key0 & 255)) * a.num_kv_heads + hkv) *
+            const int64_t e = (((static_cast<int64_t>(ok ? blk : 0) << a.block_shift) + (key0 & ((1 << a.block_shift) - 1))) * a.num_kv_heads + hkv) *
                               kHeadDim * 2;
             t.kb = reinterpret_cast<const char *>(a.k_cache) + e;
             t.vb = reinterpret_cast<const char *>(a.v_cache) + e;
@@ -532,11 +533,11 @@ extern "C" int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride, cons
     const bool paged = block_tables != nullptr;
     const int64_t dkv = static_cast<int64_t>(num_kv_heads) * head_dim;
     if (paged) {
-        if (block_size != kBlockSize) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+        if (block_shift_of(block_size) < 0) return NVA_ERR_UNSUPPORTED_GEOMETRY;
         if (!k_cache || !v_cache) return NVA_ERR_NULL_POINTER;
         if (max_blocks <= 0 || num_blocks <= 0) return NVA_ERR_BAD_SHAPE;
         if (bt_row_stride < max_blocks) return NVA_ERR_BAD_STRIDE;
-        if (static_cast<int64_t>(max_blocks) * kBlockSize < max_seqlen_k) return NVA_ERR_BAD_SHAPE;
+        if (static_cast<int64_t>(max_blocks) * block_size < max_seqlen_k) return NVA_ERR_BAD_SHAPE;
         if (!aligned16(k_cache) || !aligned16(v_cache)) return NVA_ERR_MISALIGNED;
     } else {
         if (!k || !v) return NVA_ERR_NULL_POINTER;
@@ -557,6 +558,7 @@ extern "C" int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride, cons
     a.cu_seqlens_q = cu_seqlens_q; a.cu_seqlens_k = cu_seqlens_k;
     a.out = static_cast<bf16_t *>(out);
     a.num_heads = num_heads; a.num_kv_heads = num_kv_heads; a.num_blocks = num_blocks;
+    a.block_shift = paged ? block_shift_of(block_size) : 8;
     a.scale_log2e = scale * 1.4426950408889634f;
     a.num_q_tiles = (max_seqlen_q + kPfBM - 1) / kPfBM;
     if (static_cast<int64_t>(a.num_q_tiles) * num_heads * batch > 0x7fffffffLL) return NVA_ERR_BAD_SHAPE;

@@ -84,6 +84,7 @@ def test_decode_validation_and_workspace_size():
     assert call(bt=None) == _lib.ERR_NULL_POINTER
     assert call(dh=64) == _lib.ERR_UNSUPPORTED_GEOMETRY
     assert call(bs=128) == _lib.ERR_UNSUPPORTED_GEOMETRY
+    assert call(bs=768) == _lib.ERR_UNSUPPORTED_GEOMETRY             # blocks of 256 * 2^k tokens only
     assert call(hq=72, hkv=8) == _lib.ERR_UNSUPPORTED_GEOMETRY        # group 9 (1 to 8 are built)
     assert call(hq=16, hkv=3) == _lib.ERR_UNSUPPORTED_GEOMETRY
     assert call(qs=1024) == _lib.ERR_BAD_STRIDE
@@ -120,7 +121,7 @@ def test_prefill_validation():
     assert call(out=A + 8) == _lib.ERR_MISALIGNED
     paged = dict(k=None, v=None, kc=A, vc=A, bt=A, bts=4, mb=4, nb=32)
     assert call(**dict(paged, kc=None)) == _lib.ERR_NULL_POINTER
-    assert call(**dict(paged, bs=512)) == _lib.ERR_UNSUPPORTED_GEOMETRY
+    assert call(**dict(paged, bs=768)) == _lib.ERR_UNSUPPORTED_GEOMETRY   # blocks of 256 * 2^k tokens only
     assert call(**dict(paged, bts=2)) == _lib.ERR_BAD_STRIDE
     assert call(**dict(paged, mk=4 * 256 + 1)) == _lib.ERR_BAD_SHAPE   # table too narrow for max_seqlen_k
     assert call(b=0) == _lib.OK and call(mq=0) == _lib.OK

@@ -39,6 +39,15 @@ def test_decode_gqa_groups(dev, hq, hkv):
     assert_attn_close(_gpu(case, dev), _oracle(case), f"gqa {hq}/{hkv}")
 
 
+@pytest.mark.parametrize("block_size", [512, 1024, 4096])
+def test_decode_larger_kv_blocks(dev, block_size):
+    """KV blocks of 256 * 2^k tokens (nanovllm/config.py:22 allows multiples of 256)."""
+    case = synthetic.decode_case(seed=block_size, batch=7, num_blocks=max(8, 16384 // block_size * 2), ctx_lo=1,
+                                 ctx_hi=3000, block_size=block_size)
+    assert case.k_cache.shape[1] == block_size
+    assert_attn_close(_gpu(case, dev), _oracle(case), f"block size {block_size}")
+
+
 def test_decode_edge_context_lengths(dev):
     lens = [0, 1, 2, 63, 64, 65, 255, 256, 257, 511, 512, 513, 1024, 0, 3]
     case = synthetic.decode_case(seed=7, num_blocks=64, context_lens=lens)

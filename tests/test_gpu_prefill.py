@@ -49,6 +49,17 @@ def test_prefill_config3_prefix_cache(dev):
     assert_attn_close(out, want, "config 3")
 
 
+@pytest.mark.parametrize("block_size", [512, 1024])
+def test_prefill_larger_kv_blocks(dev, block_size):
+    """KV blocks of 256 * 2^k tokens (nanovllm/config.py:22 allows multiples of 256): prefix blocks and the
+    new tokens' slots follow the larger block."""
+    case = synthetic.prefill_case(seed=block_size, batch=6, num_blocks=40, q_lo=50, q_hi=900, max_prefix_blocks=2,
+                                  block_size=block_size)
+    assert case.k_cache.shape[1] == block_size and any(case.prefix_lens)
+    out, want = _paged(case, dev)
+    assert_attn_close(out, want, f"block size {block_size}")
+
+
 @pytest.mark.parametrize("strided_v", [False, True])
 def test_prefill_no_prefix_packed(dev, strided_v):
     case = synthetic.prefill_case(seed=1, batch=6, prefix_fraction=0.0, q_lo=1, q_hi=700)
