@@ -277,7 +277,7 @@ def bench_sampler(args, dev):
                    "batch": batch},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": ("sampler_chunk_kernel<1, true>" if with_noise else "sampler_chunk_kernel<4, false>") + " + sampler_row_kernel",
+                     "kernel": ("sampler_chunk_kernel<2, true>" if with_noise else "sampler_chunk_kernel<4, false>") + " + sampler_row_kernel",
                      "algorithmic_bytes_per_launch": alg},
     }
 

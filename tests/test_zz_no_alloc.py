@@ -50,11 +50,19 @@ def test_sample_static_matches_sample_on_two_calls_in_a_row(dev, with_noise):
 
 
 def test_sample_static_rejects_what_does_not_fit(dev):
+    """Inputs and outputs are real tensors: a library that wrongly accepted the call would still touch only memory it may."""
     lib = _lib.load()
-    batch, vocab = 1748, 151936                                           # 1748 * 75 records > 131072
-    out = torch.full((4,), -5, dtype=torch.int64, device=dev)
-    rc = lib.nva_sample_static(0x1000, vocab, 0x1000, None, 0, 0, 0, out.data_ptr(), batch, vocab,
+    batch, vocab = 1748, 151936                                           # 1748 * 75 records of 2048 columns > 131072
+    logits = torch.zeros(batch, vocab, dtype=torch.bfloat16, device=dev)
+    temps = torch.ones(batch, device=dev)
+    out = torch.full((batch,), -5, dtype=torch.int64, device=dev)
+    rc = lib.nva_sample_static(logits.data_ptr(), vocab, temps.data_ptr(), None, 0, 0, 0, out.data_ptr(), batch, vocab,
                                torch.cuda.current_stream().cuda_stream)
     assert rc == _lib.ERR_SCRATCH_TOO_SMALL and "scratch" in _lib.status_string(rc)
     torch.cuda.synchronize()
-    assert out.tolist() == [-5] * 4                                       # nothing was launched
+    assert bool((out == -5).all())                                        # nothing was launched
+    rc = lib.nva_sample_static(logits.data_ptr(), vocab, temps.data_ptr(), None, 0, 0, 0, out.data_ptr(), 1747, vocab,
+                               torch.cuda.current_stream().cuda_stream)   # the largest batch that fits
+    assert rc == _lib.OK
+    torch.cuda.synchronize()
+    assert bool((out[:1747] >= 0).all()) and bool((out[:1747] < vocab).all()) and int(out[1747]) == -5
