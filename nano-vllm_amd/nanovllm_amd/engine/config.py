@@ -79,7 +79,7 @@ class EngineConfig:
             assert os.path.isdir(self.model), f"{self.model} is not a directory"
             self.hf_config = ModelConfig.from_json(os.path.join(self.model, "config.json"))
         assert self.kvcache_block_size % 256 == 0
-        assert self.kvcache_block_size == 256, "the attention kernels are built for 256-token KV blocks"
+        assert self.kvcache_block_size == 256, "this engine keeps Sequence.block_size = 256 like nanovllm/engine/sequence.py:15 (the kernels take 256 * 2^k)"
         assert self.tensor_parallel_size == 1, "this build runs on one GPU"
         assert self.graph_bucket_step >= 1
         self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
