@@ -273,7 +273,9 @@ def bench_sampler(args, dev):
         "metric": "sampler (%s), achieved HBM GB/s" % ("noise tensor given" if with_noise else "in-kernel randomness"),
         "value": round(gbps, 1), "unit": "GB/s",
         "ms_per_step": round(per_step_ms, 5),
-        "config": {"workload": "sampler: 256 rows x 151,936 bf16 logits, T=0.6, in-kernel randomness (tree of inverse-CDF draws, Philox uniforms)",
+        "config": {"workload": "sampler: 256 rows x 151,936 bf16 logits, T=0.6, " +
+                               ("Exp(1) noise tensor read (the reference's argmax(p / E))" if with_noise else
+                                "in-kernel randomness (tree of inverse-CDF draws, Philox uniforms)"),
                    "batch": batch},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
