@@ -497,6 +497,48 @@ def bench_copy(args, dev):
     return result, (lambda: None)
 
 
+def stream_read_us(dev, nbytes, steps=60, graph=False):
+    """Microseconds a bare streaming read of `nbytes` takes (nva_probe_stream_read: the decode kernel's access
+    discipline and nothing else), rotating through buffers that together exceed the 256 MB Infinity Cache.
+    `graph`: as one replayed hipGraph of the launches (for sizes where a Python call lasts as long as the kernel)."""
+    import torch
+    from nanovllm_amd import _lib
+    lib = _lib.load()
+    nbytes = nbytes // 16 * 16
+    n_buf = max(2, -(-(640 << 20) // nbytes))
+    bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(n_buf)]
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+    def call(b):
+        _lib.check(lib.nva_probe_stream_read(b.data_ptr(), nbytes, sink.data_ptr(), torch.cuda.current_stream().cuda_stream),
+                   "nva_probe_stream_read")
+    fns = [lambda b=b: call(b) for b in bufs]
+    if graph:
+        ms, _ = _graph_time_ms(fns, steps, 5)
+    else:
+        ms = _event_time_ms(fns, steps, 5)
+    return ms / steps * 1e3
+
+
+def bench_read_probe(args, dev):
+    """What a bare streaming read costs at the sizes of the bandwidth-bound kernels' workloads."""
+    sizes = {"scatter_config1 (read half of 31.9 MB)": 15_945_728, "sampler 256 x 151,936": 77_791_232,
+             "decode config 2": 291_000_000, "decode e2e shape": 855_318_528}
+    if getattr(args, "tokens", None):
+        sizes = {"%d bytes" % args.tokens: int(args.tokens)}
+    rows = {k: round(stream_read_us(dev, v, args.steps, graph=v < (64 << 20)), 2) for k, v in sizes.items()}
+    big = max(sizes.values())
+    us = rows[[k for k, v in sizes.items() if v == big][0]]
+    gbps = big / us / 1e3
+    result = {"metric": "bare streaming read (calibration), GB/s", "value": round(gbps, 1), "unit": "GB/s", "ms_per_step": round(us / 1e3, 5),
+              "config": {"workload": "nva_probe_stream_read over %d bytes; us per launch at the other sizes in `us_by_size`" % big,
+                         "us_by_size": rows},
+              "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "probe_stream_read_kernel",
+                           "algorithmic_bytes_per_launch": big}}
+    return result, (lambda: None)
+
+
 def fresh_prompts(prompts, pass_index, vocab=151936):
     """Prompts of the same lengths with newly drawn token ids: every timed pass must prefill prompts
     the engine has never seen (its prefix cache keeps the hashes of freed blocks), as the reference's
@@ -541,6 +583,14 @@ def collect_extra(dev, model, prompts, params):
         del result
         gc.collect()
         torch.cuda.empty_cache()
+    # what a kernel that only reads the same bytes takes (launch, first-load latency and the streaming rate
+    # of the part included): the attainable side of the HBM rooflines above
+    extra["attainable"] = {"what": "us per launch of a bare streaming read of the same bytes (nva_probe_stream_read)",
+                           "decode_config2_291MB_us": round(stream_read_us(dev, extra["decode_config2"]["algorithmic_bytes_per_launch"]), 2),
+                           "sampler_78MB_us": round(stream_read_us(dev, extra["sampler_256x151936"]["algorithmic_bytes_per_launch"]), 2),
+                           "decode_config5_shape_us": round(stream_read_us(dev, extra["decode_config5_shape"]["algorithmic_bytes_per_launch"], steps=12), 2)}
+    gc.collect()
+    torch.cuda.empty_cache()
     llm = LLM(model, enforce_eager=True, max_model_len=4096, num_kvcache_blocks=4096)
     llm.generate(fresh_prompts(prompts[:32], 9_000), params[:32])
     dt = _e2e_passes(llm, prompts, params, 1, 5_000)
@@ -690,8 +740,8 @@ def bench_longctx(args, dev):
 
 
 WORKLOADS = {"rope-scatter": bench_rope_scatter, "glue": bench_glue, "e2e": bench_e2e, "longctx": bench_longctx, "decode-e2e-shape": bench_decode_e2e_shape,
-             "decode-longctx-shape": bench_decode_longctx_shape, "copy": bench_copy, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
-DEFAULT_STEPS = {"rope-scatter": 100, "glue": 100, "e2e": 1, "longctx": 1, "decode-e2e-shape": 1, "decode-longctx-shape": 1, "copy": 50, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
+             "decode-longctx-shape": bench_decode_longctx_shape, "copy": bench_copy, "read-probe": bench_read_probe, "decode": bench_decode, "scatter": bench_scatter, "prefill": bench_prefill, "sampler": bench_sampler}
+DEFAULT_STEPS = {"rope-scatter": 100, "glue": 100, "e2e": 1, "longctx": 1, "decode-e2e-shape": 1, "decode-longctx-shape": 1, "copy": 50, "read-probe": 60, "decode": 200, "scatter": 400, "prefill": 50, "sampler": 100}
 
 
 def main():

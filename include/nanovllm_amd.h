@@ -268,6 +268,15 @@ int nva_stage_decode_inputs(void *dst, const void *src_host, int64_t nbytes, int
                             int64_t index_offset, int32_t n, const int64_t *prev_tokens, int32_t n_prev,
                             void *stream);
 
+/*
+ * Calibration, no counterpart in the reference: streams nbytes from src with the access discipline of
+ * the decode kernel (2048 wavefront workers, contiguous slices, 16-byte non-temporal loads) and keeps
+ * nothing.  Its duration is what any kernel that reads that many bytes needs at least on this GPU;
+ * bench.py reports it next to the roofline fractions.  src 16-byte aligned, nbytes % 16 == 0; sink:
+ * at least 4 writable bytes of device memory (practically never written).
+ */
+int nva_probe_stream_read(const void *src, int64_t nbytes, void *sink, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

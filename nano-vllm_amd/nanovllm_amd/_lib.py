@@ -47,6 +47,7 @@ SIGNATURES = {
     "nva_stage_decode_inputs": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _i32, _vp, _i32, _vp]),
     "nva_sample": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _u64, _u64, _vp, _vp, _sz, _i32, _i32, _vp]),
     "nva_sample_static": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _u64, _u64, _vp, _i32, _i32, _vp]),
+    "nva_probe_stream_read": (C.c_int, [_vp, _i64, _vp, _vp]),
 }
 
 _lib = None
