@@ -2,19 +2,24 @@
 //
 // Replaces flash_attn_with_kvcache as called by nanovllm/layers/attention.py:71-74.
 //
-// Work decomposition.  The unit of work is a "stage": 32 consecutive tokens of one kv head of
-// one sequence (8 KB of K + 8 KB of V; a stage never straddles a KV block: blocks hold 256 * 2^k tokens).  All
-// stages of the batch form one list ordered by (sequence, kv head, position) -- its length N
-// follows from context_lens alone, which every workgroup prefix-sums in LDS.  The launch is
-// a fixed set of W = 2048 wavefront "workers" (512 workgroups x 4) and worker w takes the
-// contiguous slice [w*N/W, (w+1)*N/W) (one stage each when N < W): every worker streams the same number of bytes
-// whatever the mix of context lengths, nothing is launched for empty table entries, and
-// the 8 XCDs (which receive workgroups round-robin) stay balanced.  The grid depends on no
-// device data, so the launch can be captured in a HIP graph and replayed with new contents.
-// The split (prefix sums, clipped lengths, first stage and slice of every worker) is left in the
-// workspace; a later launch over the same context_lens and block_tables -- the next layer of the
-// same decode step -- may start from it (decode_stream_kernel<G, true>) and then issues its first
-// loads after one 32-byte read instead of three dependent memory round trips.
+// Work decomposition.  The unit of a wavefront's work is a "stage": 32 consecutive tokens of one kv
+// head of one sequence (8 KB of K + 8 KB of V; a stage never straddles a KV block: blocks hold
+// 256 * 2^k tokens).  The K rows of one kv head are 256-byte pieces 2 KB apart in the cache
+// ([block, token, kv head, dim]); read head by head they stream 3-5 % slower than whole token rows.
+// So the four wavefronts of a workgroup work on a "quad" of stages side by side: the same 32 tokens
+// of four adjacent kv heads (HW = gcd(4, kv heads) heads x 4 / HW consecutive token ranges in
+// general), which together are whole 1 KB runs of the token rows, fetched at the same time.  All
+// quads of the batch form one list ordered by (sequence, group of HW kv heads, position) -- its
+// length N follows from context_lens alone, which every workgroup prefix-sums in LDS.  The launch
+// is a fixed set of 512 workgroups and workgroup x takes the contiguous slice [x*N/512, (x+1)*N/512)
+// (one quad each when N < 512): every wavefront streams the same number of bytes whatever the mix
+// of context lengths, nothing is launched for empty table entries, and the 8 XCDs (which receive
+// workgroups round-robin) stay balanced.  The grid depends on no device data, so the launch can be
+// captured in a HIP graph and replayed with new contents.  The split (prefix sums, clipped lengths,
+// first quad and slice of every wavefront) is left in the workspace; a later launch over the same
+// context_lens and block_tables -- the next layer of the same decode step -- may start from it
+// (decode_stream_kernel<G, true>) and then issues its first loads after one 32-byte read instead of
+// three dependent memory round trips.
 //
 // Per worker, a two-deep software pipeline over its stages:
 //   * HBM -> VGPR: a K (or V) head row is 128 bf16 = 256 B = 16 lanes x 16 B, so one dwordx4
@@ -31,17 +36,17 @@
 //     max / sum per lane, one exchange across the four 16-lane groups per stage.
 //   * O^T += V^T P^T: A = V^T through ds_read_b64_tr_b16 (LDS transpose read: 4 tokens x 16
 //     dims -> lane = dim, registers = tokens), B = P^T straight from the S^T registers.
-// When a worker leaves a (sequence, kv head) pair it either writes the final bf16 rows (it
+// When a wavefront leaves a (sequence, kv head) pair it either writes the final bf16 rows (it
 // saw all of the pair's stages) or an unnormalised partial (max, sum, o[128]) per query
 // head.  A second, small kernel (decode_merge_kernel) merges the partials of the pairs that
-// were split over several workers; the kernel boundary is the only synchronisation.  (Workers
+// were split over several wavefronts; the kernel boundary is the only synchronisation.  (Workers
 // sit on different XCDs, each with its own L2.  An in-kernel "last arriver merges" variant needs
 // device-scope fences, which write back and invalidate the XCD's L2: measured 3x slower for
 // the whole kernel.  Relaxed device-scope atomics without fences returned stale partials.)
 //
 // HBM traffic per sequence and layer: ctx * num_kv_heads * 128 * 2 B for K plus the same for
-// V (4096 B per token at 8 kv heads).  Partials: at most (W + batch*num_kv_heads) * G rows of 520 B;
-// the stored split: 64 KB of worker records, 8 bytes per sequence and 8 bytes per (sequence, kv head) pair.
+// V (4096 B per token at 8 kv heads).  Partials: at most (2048 + 4 * batch * num_kv_heads / HW) * G rows of
+// 520 B; the stored split: 64 KB of wavefront records, 8 bytes per sequence and 8 bytes per (sequence, kv head) pair.
 #include "nva_common.h"
 
 #include <math.h>
@@ -67,10 +72,12 @@ constexpr int kWaveLdsChunks = 2 * kStageTok * 16;  // K then V, in 16-byte chun
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(const u32x4_t &u) { return __builtin_bit_cast(bf16x8_t, u); }
 
-// the worker that owns stage x when n stages are split over nw <= n workers as [w*n/nw, (w+1)*n/nw)
+// the workgroup that owns quad x when n quads are split over nw <= n workgroups as [w*n/nw, (w+1)*n/nw)
 __device__ __forceinline__ int worker_of(int64_t x, int64_t n, int64_t nw) {
     return static_cast<int>(((x + 1) * nw - 1) / n);
 }
+// kv heads that the wavefronts of a workgroup take side by side: gcd(4, num_kv_heads)
+__host__ __device__ inline int heads_abreast(int hkv) { return hkv % 4 == 0 ? 4 : (hkv % 2 == 0 ? 2 : 1); }
 
 struct DecodeArgs {
     const bf16_t *q; int64_t q_row_stride;
@@ -78,10 +85,10 @@ struct DecodeArgs {
     const int32_t *block_tables; int32_t bt_row_stride;
     const int32_t *context_lens;
     bf16_t *out;
-    int32_t *pref_out;       // [batch + 1] stage-count prefix sums, written for the merge kernel
-    int32_t *ctx_out;        // [batch] clipped context lengths       } the work split, kept for later
-    int32_t *rec_out;        // [kDecWorkers][8] first stage per worker } launches over the same contexts
-    int32_t *pair_out;       // [batch * num_kv_heads][2] first partial row and number of partials of every pair
+    int32_t *pref_out;       // [batch + 1] quad-count prefix sums, written for the merge kernel
+    int32_t *ctx_out;        // [batch] clipped context lengths         } the work split, kept for later
+    int32_t *rec_out;        // [kDecWorkers][8] first quad per wavefront } launches over the same contexts
+    int32_t *pair_out;       // [batch * num_kv_heads][2] first partial slot and workgroups of every pair
     float *part_ml;          // [rows][2]
     float *part_o;           // [rows][128]
     int32_t batch, max_blocks, num_heads, num_kv_heads, num_blocks;
@@ -90,9 +97,15 @@ struct DecodeArgs {
 };
 
 // kReuse: the workspace already holds the work split of an earlier launch (kReuse = false) over
-// the same context_lens and block_tables; each worker then starts from its 32-byte record and
+// the same context_lens and block_tables; each wavefront then starts from its 32-byte record and
 // issues its first loads before anything else, instead of prefix-summing the context lengths and
 // reading the block table first.
+//
+// Quads.  HW = heads_abreast(num_kv_heads) kv heads side by side, PS = 4 / HW consecutive stages of
+// each: wavefront j of a workgroup takes kv head hg * HW + j % HW and stage pq * PS + j / HW of quad
+// (sequence b, head group hg, position pq).  A sequence of nst stages per head has
+// ceil(nst / PS) * (num_kv_heads / HW) quads; a wavefront whose stage lies past the sequence end
+// (PS > 1 only) runs the stage on zeros.
 template <int G, bool kReuse>
 __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const DecodeArgs a) {
     const int lane = threadIdx.x & 63;
@@ -100,9 +113,11 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
     const int grp = lane >> 4;     // 16-lane group: token row of a load, k-slot group of an MFMA
     const int r16 = lane & 15;     // chunk of a load; token / head / dim index of an MFMA operand
     const int hkv = a.num_kv_heads;
+    const int hw = heads_abreast(hkv), ps = 4 / hw, hgroups = hkv / hw;
+    const int jh = wave % hw, js = wave / hw;     // this wavefront's head inside the group, its stage inside the quad
 
-    // ---- stage-count prefix sums over the batch (every workgroup computes its own copy) -------
-    __shared__ int32_t sh_pref[kDecMaxBatch + 1];   // sh_pref[b] = stages of all (sequence < b, head)
+    // ---- quad-count prefix sums over the batch (every workgroup computes its own copy) --------
+    __shared__ int32_t sh_pref[kDecMaxBatch + 1];   // sh_pref[b] = quads of all sequences < b
     __shared__ int32_t sh_ctx[kDecMaxBatch];        // context length of sequence b, clipped to the table
     __shared__ __attribute__((aligned(16))) u32x4_t lds[kDecWaves * kWaveLdsChunks];
     const int w = blockIdx.x * kDecWaves + wave;
@@ -110,23 +125,33 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
     u32x4_t *sV = sK + kStageTok * 16;
     const int64_t row = static_cast<int64_t>(hkv) * kHeadDim;       // elements per token row
 
-    // Block and number of valid rows (minus one) of stage ss of sequence bb.
+    // Block and number of valid rows (minus one) of stage ss of sequence bb; last = -1 when the stage
+    // lies past the sequence end or behind a bad table entry (it then contributes nothing).
     auto locate = [&](int bb, int ss, int32_t &blk, int &last) __attribute__((always_inline)) {
-        last = min(kStageTok, sh_ctx[bb] - ss * kStageTok) - 1;                // in [0, 31]
-        blk = a.block_tables[static_cast<int64_t>(bb) * a.bt_row_stride + (ss >> (a.block_shift - 5))];
-        if (static_cast<uint32_t>(blk) >= static_cast<uint32_t>(a.num_blocks)) {
-            blk = 0;                                  // bad table entry: contributes nothing
+        last = min(kStageTok, sh_ctx[bb] - ss * kStageTok) - 1;                // <= 31
+        blk = 0;
+        if (last >= 0) {
+            blk = a.block_tables[static_cast<int64_t>(bb) * a.bt_row_stride + (ss >> (a.block_shift - 5))];
+            if (static_cast<uint32_t>(blk) >= static_cast<uint32_t>(a.num_blocks)) {
+                blk = 0;                                  // bad table entry
+                last = -1;
+            }
+        } else {
             last = -1;
         }
     };
     // HBM -> registers for stage ss of kv head gg of sequence bb, which lies in block blk.  Token
     // rows are clamped to the last valid row of the stage, so only rows that were written are touched.
+    // A stage without valid rows (last < 0) reads the sequence's own first query row instead of the
+    // cache: every score of it is masked, so any finite data will do, and unwritten cache rows may
+    // hold bit patterns that are not numbers (0 * NaN would reach the output).
     auto issue = [&](int bb, int gg, int ss, int32_t blk, int last, u32x4_t (&kr)[kStageLoads],
                      u32x4_t (&vr)[kStageLoads], u32x4_t (&qr)[4]) __attribute__((always_inline)) {
         const int tok0 = (ss << 5) & ((1 << a.block_shift) - 1);       // (kStageTok = 32 tokens per stage)
         const int64_t base = ((static_cast<int64_t>(blk) << a.block_shift) + tok0) * row + gg * kHeadDim + r16 * 8;
-        const bf16_t *kb = a.k_cache + base;
-        const bf16_t *vb = a.v_cache + base;
+        const bf16_t *qrow = a.q + static_cast<int64_t>(bb) * a.q_row_stride + r16 * 8;
+        const bf16_t *kb = last >= 0 ? a.k_cache + base : qrow;
+        const bf16_t *vb = last >= 0 ? a.v_cache + base : qrow;
         const int lastc = max(last, 0);
         // K/V are read once and never again: non-temporal loads keep them from displacing one another in L2
         // (measured +12 % bandwidth over plain loads)
@@ -146,16 +171,10 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
             qr[i] = u;
         }
     };
-    auto load_stage = [&](int bb, int gg, int ss, u32x4_t (&kr)[kStageLoads], u32x4_t (&vr)[kStageLoads],
-                          u32x4_t (&qr)[4], int &last) __attribute__((always_inline)) {
-        int32_t blk;
-        locate(bb, ss, blk, last);
-        issue(bb, gg, ss, blk, last, kr, vr, qr);
-    };
 
     u32x4_t kr[kStageLoads], vr[kStageLoads], qr[4];
-    int b, g, s, nst, last;
-    int64_t lo, hi;
+    int b, hg, pq, nqp, last;      // quad (b, hg, pq) of a sequence with nqp quads per head group
+    int64_t lo, hi;                // this workgroup's slice of the quad list
     if constexpr (kReuse) {
         // ---- the split is in the workspace: first loads first, then the tables into LDS ---------
         const int4 *rec = reinterpret_cast<const int4 *>(a.rec_out) + 2 * w;
@@ -169,9 +188,9 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
             cv[i] = at < a.batch ? a.ctx_out[at] : 0;
         }
         const int total = a.pref_out[a.batch];
-        b = r0.x; g = r0.y; s = r0.z; nst = r0.w;
+        b = r0.x; hg = r0.y; pq = r0.z; nqp = r0.w;
         last = r1.y; lo = r1.z; hi = r1.w;
-        if (nst > 0) issue(b, g, s, r1.x, last, kr, vr, qr);
+        if (nqp > 0) issue(b, hg * hw + jh, pq * ps + js, r1.x, last, kr, vr, qr);
 #pragma unroll
         for (int i = 0; i < kPer; ++i) {
             const int at = threadIdx.x + i * kDecThreads;
@@ -195,7 +214,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
                     // a context that does not fit the table is clipped to it instead of read out of bounds
                     const int ctx = min(max(a.context_lens[bi], 0), a.max_blocks << a.block_shift);
                     sh_ctx[bi] = ctx;
-                    c = (ctx + kStageTok - 1) / kStageTok * hkv;
+                    c = ((ctx + kStageTok - 1) / kStageTok + ps - 1) / ps * hgroups;
                 }
                 cnt[i] = c;
                 local += c;
@@ -231,21 +250,21 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
     }
 
     if constexpr (kReuse) {
-        if (nst == 0) return;                            // idle worker (wave-uniform; no barrier follows)
+        if (nqp == 0) return;                            // idle workgroup (uniform; no barrier follows)
     } else {
-        // With fewer stages than workers only the first n_total workers get (one) stage each, so that
-        // the workers of a pair are always consecutive.
+        // With fewer quads than workgroups only the first n_total workgroups get (one) quad each, so that
+        // the workgroups of a pair are always consecutive.
         const int64_t n_total = sh_pref[a.batch];
-        const int64_t n_workers = n_total < kDecWorkers ? n_total : kDecWorkers;
+        const int64_t n_wgs = n_total < kDecGrid ? n_total : kDecGrid;
         int4 *rec = reinterpret_cast<int4 *>(a.rec_out) + 2 * w;
-        if (w >= n_workers) {                            // wave-uniform; no barrier follows
+        if (blockIdx.x >= n_wgs) {                       // uniform over the workgroup; no barrier follows
             if (lane == 0) rec[0] = int4{0, 0, 0, 0};
             return;
         }
-        lo = static_cast<int64_t>(w) * n_total / n_workers;
-        hi = static_cast<int64_t>(w + 1) * n_total / n_workers;   // > lo
+        lo = static_cast<int64_t>(blockIdx.x) * n_total / n_wgs;
+        hi = static_cast<int64_t>(blockIdx.x + 1) * n_total / n_wgs;   // > lo
 
-        // ---- locate the first stage: largest b with sh_pref[b] <= lo ----------------------------
+        // ---- locate the first quad: largest b with sh_pref[b] <= lo -----------------------------
         {
             int l = 0, r = a.batch;                      // invariant: sh_pref[l] <= lo < sh_pref[r]
             while (r - l > 1) {
@@ -254,14 +273,14 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
             }
             b = l;
         }
-        nst = (sh_pref[b + 1] - sh_pref[b]) / hkv;       // stages per head of sequence b (> 0)
-        g = static_cast<int>(lo - sh_pref[b]) / nst;
-        s = static_cast<int>(lo - sh_pref[b]) % nst;
+        nqp = (sh_pref[b + 1] - sh_pref[b]) / hgroups;   // quads per head group of sequence b (> 0)
+        hg = static_cast<int>(lo - sh_pref[b]) / nqp;
+        pq = static_cast<int>(lo - sh_pref[b]) % nqp;
         int32_t blk;
-        locate(b, s, blk, last);
-        issue(b, g, s, blk, last, kr, vr, qr);
+        locate(b, pq * ps + js, blk, last);
+        issue(b, hg * hw + jh, pq * ps + js, blk, last, kr, vr, qr);
         if (lane == 0) {
-            rec[0] = int4{b, g, s, nst};
+            rec[0] = int4{b, hg, pq, nqp};
             rec[1] = int4{blk, last, static_cast<int>(lo), static_cast<int>(hi)};
         }
     }
@@ -275,6 +294,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
         l_run = 0.f;
     };
     reset_state();
+    const int64_t part_stride = kDecGrid + static_cast<int64_t>(a.batch) * hgroups;   // partial slots of one wavefront index
 
     for (int64_t x = lo; x < hi; ++x) {
         // ---- registers -> LDS (swizzled) ------------------------------------------------------
@@ -288,26 +308,28 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
 #pragma unroll
         for (int i = 0; i < 4; ++i) qf[i] = as_bf16x8(qr[i]);
         const int cur_last = last;
-        const int cur_b = b, cur_g = g, cur_nst = nst;
+        const int cur_b = b, cur_hg = hg, cur_nqp = nqp;
 
-        // ---- coordinates of the next stage; its loads fly during this stage's arithmetic ------
+        // ---- coordinates of the next quad; its loads fly during this stage's arithmetic -------
         const bool more = x + 1 < hi;
         bool pair_ends = true;
         if (more) {
-            if (s + 1 < nst) {
-                ++s;
+            if (pq + 1 < nqp) {
+                ++pq;
                 pair_ends = false;
             } else {
-                s = 0;
-                if (g + 1 < hkv) {
-                    ++g;
+                pq = 0;
+                if (hg + 1 < hgroups) {
+                    ++hg;
                 } else {
-                    g = 0;
+                    hg = 0;
                     do { ++b; } while (sh_pref[b + 1] == sh_pref[b]);   // skip sequences without keys
-                    nst = (sh_pref[b + 1] - sh_pref[b]) / hkv;
+                    nqp = (sh_pref[b + 1] - sh_pref[b]) / hgroups;
                 }
             }
-            load_stage(b, g, s, kr, vr, qr, last);
+            int32_t blk;
+            locate(b, pq * ps + js, blk, last);
+            issue(b, hg * hw + jh, pq * ps + js, blk, last, kr, vr, qr);
         }
         __builtin_amdgcn_wave_barrier();
 
@@ -377,13 +399,14 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
         }
         __builtin_amdgcn_wave_barrier();               // this stage's LDS reads precede the next stage's writes
 
-        // ---- leaving the (sequence, kv head) pair: final rows, or a partial for the merge --------
+        // ---- leaving the (sequence, head group): final rows, or a partial for the merge -----------
         if (pair_ends) {
             float l_tot = l_run + __shfl_xor(l_run, 16, 64);
             l_tot += __shfl_xor(l_tot, 32, 64);
-            const int64_t pair_lo = sh_pref[cur_b] + static_cast<int64_t>(cur_g) * cur_nst;   // first stage of the pair
-            const int64_t pair_hi = pair_lo + cur_nst;
-            if (lo <= pair_lo && pair_hi <= hi) {      // this worker saw the whole pair
+            const int cur_g = cur_hg * hw + jh;
+            const int64_t pair_lo = sh_pref[cur_b] + static_cast<int64_t>(cur_hg) * cur_nqp;   // first quad of the head group
+            const int64_t pair_hi = pair_lo + cur_nqp;
+            if (ps == 1 && lo <= pair_lo && pair_hi <= hi) {      // this wavefront saw the whole pair
                 if (r16 < G) {
                     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
                     bf16_t *op = a.out + (static_cast<int64_t>(cur_b) * a.num_heads + cur_g * G + r16) * kHeadDim + 4 * grp;
@@ -395,8 +418,8 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
                     }
                 }
             } else {
-                const int pair = cur_b * hkv + cur_g;
-                const int64_t slot = static_cast<int64_t>(w) + pair;   // unique per (worker, pair) along the stage list
+                // unique per (workgroup, head group) along the quad list, one range of slots per wavefront index
+                const int64_t slot = wave * part_stride + blockIdx.x + (static_cast<int64_t>(cur_b) * hgroups + cur_hg);
                 if (r16 < G) {
                     float *po = a.part_o + (slot * G + r16) * kHeadDim + 4 * grp;
 #pragma unroll
@@ -412,13 +435,15 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
     }
 }
 
-// Merges the partials of every (sequence, kv head) pair that was split over several workers.
+// Merges the partials of every (sequence, kv head) pair that was split over several wavefronts.
 // One workgroup of G wavefronts per pair: wavefront h merges query head g*G + h, lane = 2 dims.
-// Which workers met the pair follows from the stage-count prefix sums the streaming kernel left in
-// the workspace; pairs seen by a single worker were already written.  The building call also leaves
-// (first partial row, number of partials) per pair in the workspace, so that a call that reuses the
-// work split starts from one 8-byte read instead of three dependent ones.  The partials of a pair
-// are fetched eight at a time, all loads of a round in flight together.
+// Which workgroups met the pair's head group follows from the quad-count prefix sums the streaming
+// kernel left in the workspace; a pair seen by a single wavefront was already written.  The partials
+// of the pair are the rows (j * stride + slot0 + i) * G + h for the 4 / HW wavefront indices j that
+// carry its kv head and i = 0 .. workgroups - 1.  The building call also leaves (slot0, workgroups)
+// per pair in the workspace, so that a call that reuses the work split starts from one 8-byte read
+// instead of three dependent ones.  The partials are fetched eight at a time, all loads of a round
+// in flight together.
 template <int G, bool kReuse>
 __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArgs a) {
     const int pair = blockIdx.x;
@@ -426,36 +451,45 @@ __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArg
     const int g = pair % a.num_kv_heads;
     const int h = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
-    int64_t row0;
-    int n_parts;
+    const int hw = heads_abreast(a.num_kv_heads), ps = 4 / hw, hgroups = a.num_kv_heads / hw;
+    const int64_t part_stride = kDecGrid + static_cast<int64_t>(a.batch) * hgroups;
+    int64_t slot0;
+    int n_wgs;
     if constexpr (kReuse) {
         const int2 info = reinterpret_cast<const int2 *>(a.pair_out)[pair];
-        row0 = static_cast<int64_t>(info.x) + h;
-        n_parts = info.y;
+        slot0 = info.x;
+        n_wgs = info.y;
     } else {
         const int64_t n_total = a.pref_out[a.batch];
         const int pb = a.pref_out[b];
-        const int nst = (a.pref_out[b + 1] - pb) / a.num_kv_heads;
-        n_parts = 0;                                   // no keys: the zero rows are already there
-        row0 = 0;
-        if (nst > 0) {
-            const int64_t n_workers = n_total < kDecWorkers ? n_total : kDecWorkers;
-            const int64_t pair_lo = pb + static_cast<int64_t>(g) * nst;
-            const int w_first = worker_of(pair_lo, n_total, n_workers);
-            n_parts = worker_of(pair_lo + nst - 1, n_total, n_workers) - w_first + 1;
-            row0 = (static_cast<int64_t>(w_first) + pair) * G;   // rows of consecutive workers are G apart
+        const int nqp = (a.pref_out[b + 1] - pb) / hgroups;
+        n_wgs = 0;                                     // no keys: the zero rows are already there
+        slot0 = 0;
+        if (nqp > 0) {
+            const int64_t grid = n_total < kDecGrid ? n_total : kDecGrid;
+            const int hg = g / hw;
+            const int64_t pair_lo = pb + static_cast<int64_t>(hg) * nqp;
+            const int x_first = worker_of(pair_lo, n_total, grid);
+            n_wgs = worker_of(pair_lo + nqp - 1, n_total, grid) - x_first + 1;
+            slot0 = static_cast<int64_t>(x_first) + static_cast<int64_t>(b) * hgroups + hg;   // slots of consecutive workgroups are consecutive
         }
-        if (threadIdx.x == 0) reinterpret_cast<int2 *>(a.pair_out)[pair] = int2{static_cast<int>(row0), n_parts};
-        row0 += h;
+        if (threadIdx.x == 0) reinterpret_cast<int2 *>(a.pair_out)[pair] = int2{static_cast<int>(slot0), n_wgs};
     }
-    if (n_parts <= 1) return;                          // one worker saw the whole pair and wrote it
+    const int n_parts = n_wgs * ps;
+    if (n_parts <= 1) return;                          // one wavefront saw the whole pair and wrote it
+    const int jh = g % hw;
+    // partial t of the pair: wavefront index jh + hw * (t / n_wgs), workgroup t % n_wgs of the pair's run
+    auto part_row = [&](int t) __attribute__((always_inline)) -> int64_t {
+        const int js = t / n_wgs;
+        return ((jh + hw * js) * part_stride + slot0 + (t - js * n_wgs)) * G + h;
+    };
     float mx = -INFINITY, lsum = 0.f, acc0 = 0.f, acc1 = 0.f;
     for (int base = 0; base < n_parts; base += 8) {
         float pm[8], pl[8];
         float2 po[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const int64_t at = row0 + static_cast<int64_t>(min(base + j, n_parts - 1)) * G;
+            const int64_t at = part_row(min(base + j, n_parts - 1));
             const float2 ml = *reinterpret_cast<const float2 *>(a.part_ml + at * 2);
             po[j] = *reinterpret_cast<const float2 *>(a.part_o + at * kHeadDim + 2 * lane);
             pm[j] = base + j < n_parts ? ml.x : -INFINITY;
@@ -471,7 +505,7 @@ __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArg
             acc1 *= keep;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const float f = exp2f(pm[j] - m_new);  // 0 for slots past the last partial
+                const float f = exp2f(pm[j] - m_new);  // 0 for slots past the last partial and for partials without keys
                 lsum = fmaf(f, pl[j], lsum);
                 acc0 = fmaf(f, po[j].x, acc0);
                 acc1 = fmaf(f, po[j].y, acc1);
@@ -507,9 +541,11 @@ static DecodeWorkspace decode_workspace(int32_t batch, int32_t num_heads, int32_
     DecodeWorkspace ws;
     const size_t per_launch = static_cast<size_t>(batch < kDecMaxBatch ? batch : kDecMaxBatch);
     ws.pref_bytes = align_up((per_launch + 1) * sizeof(int32_t), 256);
-    // partial rows: one per query head of every (worker, pair) met along the stage list;
-    // row index = (worker + pair) * G + head < W * G + batch * num_heads, and G <= 8
-    ws.rows = static_cast<size_t>(kDecWorkers) * (num_heads < 8 ? num_heads : 8) + per_launch * num_heads;
+    // partial rows: one per query head of every (wavefront, head group) met along the quad list;
+    // row index = (j * (512 + batch * head groups) + workgroup + sequence * head groups + head group) * G + head
+    // with j < 4, i.e. below 2048 * G + 4 * batch * num_heads / HW; G <= 8 and HW >= 1 (the size does not depend on
+    // the number of kv heads: the caller sizes the workspace without it)
+    ws.rows = static_cast<size_t>(kDecWorkers) * (num_heads < 8 ? num_heads : 8) + 4 * per_launch * num_heads;
     ws.ctx_bytes = align_up(per_launch * sizeof(int32_t), 256);
     ws.rec_bytes = static_cast<size_t>(kDecWorkers) * 8 * sizeof(int32_t);
     ws.pair_bytes = align_up(per_launch * static_cast<size_t>(num_kv_heads) * 2 * sizeof(int32_t), 256);
