@@ -93,6 +93,8 @@ struct DecodeArgs {
     float *part_o;           // [rows][128]
     int32_t batch, max_blocks, num_heads, num_kv_heads, num_blocks;
     int32_t block_shift;     // log2 of the tokens per KV block (256, 512, ... : a power of two)
+    int32_t hw, hw_shift;    // kv heads taken side by side by the wavefronts of a workgroup (1, 2 or 4) and its log2
+    int32_t hgroups;         // num_kv_heads / hw
     float scale_log2e;
 };
 
@@ -113,8 +115,8 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
     const int grp = lane >> 4;     // 16-lane group: token row of a load, k-slot group of an MFMA
     const int r16 = lane & 15;     // chunk of a load; token / head / dim index of an MFMA operand
     const int hkv = a.num_kv_heads;
-    const int hw = heads_abreast(hkv), ps = 4 / hw, hgroups = hkv / hw;
-    const int jh = wave % hw, js = wave / hw;     // this wavefront's head inside the group, its stage inside the quad
+    const int hw = a.hw, ps = 4 >> a.hw_shift, hgroups = a.hgroups;
+    const int jh = wave & (hw - 1), js = wave >> a.hw_shift;     // this wavefront's head inside the group, its stage inside the quad
 
     // ---- quad-count prefix sums over the batch (every workgroup computes its own copy) --------
     __shared__ int32_t sh_pref[kDecMaxBatch + 1];   // sh_pref[b] = quads of all sequences < b
@@ -214,7 +216,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
                     // a context that does not fit the table is clipped to it instead of read out of bounds
                     const int ctx = min(max(a.context_lens[bi], 0), a.max_blocks << a.block_shift);
                     sh_ctx[bi] = ctx;
-                    c = ((ctx + kStageTok - 1) / kStageTok + ps - 1) / ps * hgroups;
+                    c = (((ctx + kStageTok - 1) / kStageTok + ps - 1) >> (2 - a.hw_shift)) * hgroups;
                 }
                 cnt[i] = c;
                 local += c;
@@ -294,7 +296,6 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
         l_run = 0.f;
     };
     reset_state();
-    const int64_t part_stride = kDecGrid + static_cast<int64_t>(a.batch) * hgroups;   // partial slots of one wavefront index
 
     for (int64_t x = lo; x < hi; ++x) {
         // ---- registers -> LDS (swizzled) ------------------------------------------------------
@@ -418,8 +419,8 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
                     }
                 }
             } else {
-                // unique per (workgroup, head group) along the quad list, one range of slots per wavefront index
-                const int64_t slot = wave * part_stride + blockIdx.x + (static_cast<int64_t>(cur_b) * hgroups + cur_hg);
+                // (workgroup + head group) is unique per (workgroup, head group) along the quad list; its four wavefronts' rows are neighbours
+                const int64_t slot = (blockIdx.x + (static_cast<int64_t>(cur_b) * hgroups + cur_hg)) * kDecWaves + wave;
                 if (r16 < G) {
                     float *po = a.part_o + (slot * G + r16) * kHeadDim + 4 * grp;
 #pragma unroll
@@ -439,7 +440,7 @@ __global__ __launch_bounds__(kDecThreads, 2) void decode_stream_kernel(const Dec
 // One workgroup of G wavefronts per pair: wavefront h merges query head g*G + h, lane = 2 dims.
 // Which workgroups met the pair's head group follows from the quad-count prefix sums the streaming
 // kernel left in the workspace; a pair seen by a single wavefront was already written.  The partials
-// of the pair are the rows (j * stride + slot0 + i) * G + h for the 4 / HW wavefront indices j that
+// of the pair are the rows ((slot0 + i) * 4 + j) * G + h for the 4 / HW wavefront indices j that
 // carry its kv head and i = 0 .. workgroups - 1.  The building call also leaves (slot0, workgroups)
 // per pair in the workspace, so that a call that reuses the work split starts from one 8-byte read
 // instead of three dependent ones.  The partials are fetched eight at a time, all loads of a round
@@ -451,8 +452,7 @@ __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArg
     const int g = pair % a.num_kv_heads;
     const int h = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
-    const int hw = heads_abreast(a.num_kv_heads), ps = 4 / hw, hgroups = a.num_kv_heads / hw;
-    const int64_t part_stride = kDecGrid + static_cast<int64_t>(a.batch) * hgroups;
+    const int hw = a.hw, ps = 4 >> a.hw_shift, hgroups = a.hgroups;
     int64_t slot0;
     int n_wgs;
     if constexpr (kReuse) {
@@ -467,7 +467,7 @@ __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArg
         slot0 = 0;
         if (nqp > 0) {
             const int64_t grid = n_total < kDecGrid ? n_total : kDecGrid;
-            const int hg = g / hw;
+            const int hg = g >> a.hw_shift;
             const int64_t pair_lo = pb + static_cast<int64_t>(hg) * nqp;
             const int x_first = worker_of(pair_lo, n_total, grid);
             n_wgs = worker_of(pair_lo + nqp - 1, n_total, grid) - x_first + 1;
@@ -477,11 +477,11 @@ __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArg
     }
     const int n_parts = n_wgs * ps;
     if (n_parts <= 1) return;                          // one wavefront saw the whole pair and wrote it
-    const int jh = g % hw;
+    const int jh = g & (hw - 1);
     // partial t of the pair: wavefront index jh + hw * (t / n_wgs), workgroup t % n_wgs of the pair's run
     auto part_row = [&](int t) __attribute__((always_inline)) -> int64_t {
-        const int js = t / n_wgs;
-        return ((jh + hw * js) * part_stride + slot0 + (t - js * n_wgs)) * G + h;
+        const int js = (t >= n_wgs) + (t >= 2 * n_wgs) + (t >= 3 * n_wgs);     // t / n_wgs, which is below 4
+        return ((slot0 + (t - js * n_wgs)) * kDecWaves + (jh + hw * js)) * G + h;
     };
     float mx = -INFINITY, lsum = 0.f, acc0 = 0.f, acc1 = 0.f;
     for (int base = 0; base < n_parts; base += 8) {
@@ -542,7 +542,7 @@ static DecodeWorkspace decode_workspace(int32_t batch, int32_t num_heads, int32_
     const size_t per_launch = static_cast<size_t>(batch < kDecMaxBatch ? batch : kDecMaxBatch);
     ws.pref_bytes = align_up((per_launch + 1) * sizeof(int32_t), 256);
     // partial rows: one per query head of every (wavefront, head group) met along the quad list;
-    // row index = (j * (512 + batch * head groups) + workgroup + sequence * head groups + head group) * G + head
+    // row index = ((workgroup + sequence * head groups + head group) * 4 + j) * G + head
     // with j < 4, i.e. below 2048 * G + 4 * batch * num_heads / HW; G <= 8 and HW >= 1 (the size does not depend on
     // the number of kv heads: the caller sizes the workspace without it)
     ws.rows = static_cast<size_t>(kDecWorkers) * (num_heads < 8 ? num_heads : 8) + 4 * per_launch * num_heads;
@@ -625,6 +625,9 @@ extern "C" int nva_paged_decode_attn_planned(const void *q, int64_t q_row_stride
     a.num_kv_heads = num_kv_heads;
     a.num_blocks = num_blocks;
     a.block_shift = block_shift;
+    a.hw = heads_abreast(num_kv_heads);
+    a.hw_shift = a.hw == 4 ? 2 : (a.hw == 2 ? 1 : 0);
+    a.hgroups = num_kv_heads / a.hw;
     a.scale_log2e = scale * 1.4426950408889634f;
     // launches of at most kDecMaxBatch sequences each, back to back on the stream
     for (int32_t b0 = 0; b0 < batch; b0 += kDecMaxBatch) {
