@@ -479,9 +479,11 @@ __global__ __launch_bounds__(G * kWave) void decode_merge_kernel(const DecodeArg
     if (n_parts <= 1) return;                          // one wavefront saw the whole pair and wrote it
     const int jh = g & (hw - 1);
     // partial t of the pair: wavefront index jh + hw * (t / n_wgs), workgroup t % n_wgs of the pair's run
+    const int64_t row_first = (slot0 * kDecWaves + jh) * G + h;               // partial 0; consecutive workgroups are 4 G rows apart
     auto part_row = [&](int t) __attribute__((always_inline)) -> int64_t {
+        if (ps == 1) return row_first + static_cast<int64_t>(t) * (kDecWaves * G);   // (the usual case: kv heads a multiple of 4)
         const int js = (t >= n_wgs) + (t >= 2 * n_wgs) + (t >= 3 * n_wgs);     // t / n_wgs, which is below 4
-        return ((slot0 + (t - js * n_wgs)) * kDecWaves + (jh + hw * js)) * G + h;
+        return row_first + (static_cast<int64_t>(t - js * n_wgs) * kDecWaves + hw * js) * G;
     };
     float mx = -INFINITY, lsum = 0.f, acc0 = 0.f, acc1 = 0.f;
     for (int base = 0; base < n_parts; base += 8) {
