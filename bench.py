@@ -15,12 +15,14 @@ already resident in HBM.  Workloads (shapes are the five benchmark configuration
     glue      residual add + RMSNorm (--glue add-rms-norm) or SiLU(gate) * up (--glue silu-mul), 16,384 rows (--tokens N)
     decode-e2e-shape / decode-longctx-shape / copy   profiling helpers: the decode attention of configs 4 / 5
               alone (one layer); a plain copy of known size
+    read-probe    calibration: a bare streaming read at the sizes of the bandwidth-bound workloads
 The line carries `roofline` (algorithmic bytes or flops of the dominant kernel per launch,
 divided by its average duration measured with HIP events on the launch stream) and
 `cpu_baseline` (the CPU oracle timed on this box's host cores on a bounded sample).  The default
 (e2e) line also carries `extra`: the rooflines of the scatter, decode, prefill and sampler
 configurations and of the long-context decode shape, each timed in isolation in the same run, and
-one eager (no hipGraph) pass of the same workload.  Every timed e2e pass generates from prompts
+one eager (no hipGraph) pass of the same workload, and `extra.attainable`: what a bare streaming read of the decode and
+sampler workloads' bytes takes on this GPU.  Every timed e2e pass generates from prompts
 the engine has not seen (fresh draw per pass), like the reference's bench.py:22-27.
 The scatter workload is timed as one replayed hipGraph of its K launches (a Python call costs as much
 as that 7 us kernel; the eager-loop figure is reported beside it).
