@@ -67,9 +67,9 @@ def test_decode_validation_and_workspace_size():
     lib = _lib.load()
     ws = lib.nva_paged_decode_workspace_bytes
     # prefix sums and context lengths (each 256-byte aligned) + a 32-byte record per worker + 8 bytes per
-    # (sequence, head) pair (256-byte aligned) + (2048 workers * min(heads, 8) + batch * heads) partial rows of 130 floats
-    assert ws(64, 16, 128, 8) == 512 + 256 + 2048 * 32 + 64 * 16 * 8 + (2048 * 8 + 64 * 16) * 130 * 4
-    assert ws(3, 2, 128, 1) == 256 + 256 + 2048 * 32 + 256 + (2048 * 2 + 3 * 2) * 130 * 4
+    # (sequence, head) pair (256-byte aligned) + (2048 wavefronts * min(heads, 8) + 4 * batch * heads) partial rows of 130 floats
+    assert ws(64, 16, 128, 8) == 512 + 256 + 2048 * 32 + 64 * 16 * 8 + (2048 * 8 + 4 * 64 * 16) * 130 * 4
+    assert ws(3, 2, 128, 1) == 256 + 256 + 2048 * 32 + 256 + (2048 * 2 + 4 * 3 * 2) * 130 * 4
     assert ws(0, 16, 128, 8) == 0
     f = lib.nva_paged_decode_attn
     ok = dict(q=A, qs=2048, kc=A, vc=A, bt=A, bts=8, mb=8, cl=A, out=A, ws=A, wsb=ws(4, 16, 128, 8),
@@ -189,3 +189,15 @@ def test_sample_static_validation():
     assert f(A, 100, A, None, 0, 0, 0, A, 0, 100, None) == _lib.OK
     assert f(A, 151936, A, None, 0, 0, 0, A, 1748, 151936, None) == _lib.ERR_SCRATCH_TOO_SMALL    # 1748 * 75 records > 131072
     assert f(A, 1 << 29, A, None, 0, 0, 0, A, 1, 1 << 29, None) == _lib.ERR_SCRATCH_TOO_SMALL     # 262144 records
+
+
+def test_probe_validation():
+    """The calibration read rejects bad arguments before any launch."""
+    f = _lib.load().nva_probe_stream_read
+    # (src, nbytes, sink, stream)
+    assert f(None, 1024, A, None) == _lib.ERR_NULL_POINTER
+    assert f(A, 1024, None, None) == _lib.ERR_NULL_POINTER
+    assert f(A + 8, 1024, A, None) == _lib.ERR_MISALIGNED
+    assert f(A, 1000, A, None) == _lib.ERR_MISALIGNED               # not a multiple of 16
+    assert f(A, -16, A, None) == _lib.ERR_BAD_SHAPE
+    assert f(A, 0, A, None) == _lib.OK                               # nothing to read

@@ -78,3 +78,17 @@ def test_scatter_out_of_range_slots_are_skipped(dev):
     keep[::2] = -1
     oracle.store_kvcache(case.key, case.value, ek, ev, keep)
     assert torch.equal(bits(kc), bits(ek)) and torch.equal(bits(vc), bits(ev))
+
+
+def test_calibration_read_touches_nothing(dev):
+    """nva_probe_stream_read only reads: the source is unchanged and the sink keeps its value."""
+    from nanovllm_amd import _lib
+    lib = _lib.load()
+    src = torch.randint(0, 255, (3 * 1024 * 1024 + 48,), dtype=torch.uint8, device=dev)
+    before = src.clone()
+    sink = torch.full((4,), 7, dtype=torch.int32, device=dev)
+    for nbytes in (16, 4096 + 16, src.numel()):
+        rc = lib.nva_probe_stream_read(src.data_ptr(), nbytes, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == _lib.OK
+    torch.cuda.synchronize()
+    assert torch.equal(src, before) and sink.tolist() == [7] * 4
