@@ -32,7 +32,8 @@ def test_decode_config2(dev):
     assert_attn_close(out, _oracle(case), "config 2")
 
 
-@pytest.mark.parametrize("hq,hkv", [(32, 8), (8, 8), (16, 2), (8, 1), (24, 8), (40, 8), (12, 2), (7, 1)])   # groups 4 1 8 8 3 5 6 7
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (8, 8), (16, 2), (8, 1), (24, 8), (40, 8), (12, 2), (7, 1),   # groups 4 1 8 8 3 5 6 7
+                                    (6, 3), (12, 6), (10, 5), (12, 12)])                                     # kv heads that are no multiple of 4: 1 or 2 heads side by side
 def test_decode_gqa_groups(dev, hq, hkv):
     case = synthetic.decode_case(seed=hq * 10 + hkv, batch=9, num_heads=hq, num_kv_heads=hkv, num_blocks=64,
                                  ctx_lo=1, ctx_hi=1200)
