@@ -8,8 +8,9 @@
  * with the *_workspace_bytes functions).  Arguments are validated on the host before any
  * launch; a non-zero return means nothing was enqueued.
  *
- * Dtypes / geometry: bf16 tensors, int32 index tensors, head_dim 128, KV block size 256,
- * num_heads / num_kv_heads from 1 to 8.  Anything else is rejected with
+ * Dtypes / geometry: bf16 tensors, int32 index tensors, head_dim 128, KV blocks of 256, 512,
+ * 1024, 2048 or 4096 tokens, num_heads / num_kv_heads from 1 to 8 (decode; prefill takes any
+ * multiple).  Anything else is rejected with
  * NVA_ERR_UNSUPPORTED_GEOMETRY rather than served by a slow path.
  *
  * File:line citations name the reference (nano-vllm) interface each entry point replaces.
@@ -158,7 +159,7 @@ int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride,
  * temperatures: fp32 [batch].  T == 0 selects greedy argmax(logits) for that row (an
  * extension; the reference forbids T <= 1e-10, nanovllm/sampling_params.py:11).
  * noise: fp32 [batch, vocab] Exp(1) draws (row stride noise_row_stride): the formula above is
- * evaluated (scores relative to the maximum of each 2048-column chunk, rescaled to the row) and a
+ * evaluated (scores relative to the maximum of each 4096-column chunk, rescaled to the row) and a
  * draw can be replayed; the argmax differs from the formula only between scores that agree to fp32
  * rounding.  NULL: the token is drawn from the same categorical distribution softmax(logits / T) by a
  * tree of inverse-CDF steps (row -> chunk of 8192 columns -> one of 4 column groups -> one of its 64
@@ -167,7 +168,9 @@ int nva_varlen_prefill_attn(const void *q, int64_t q_row_stride,
  * (seed, offset, row, chunk); the same (seed, offset) reproduces the draw.  Sums are fp32 and a
  * conditional probability below 2^-32 at a level is not resolved.
  * out_tokens: int64 [batch].
- * workspace: at least nva_sample_workspace_bytes() bytes, 16-byte aligned.
+ * workspace: at least nva_sample_workspace_bytes() bytes, 16-byte aligned.  Its size (and the limit
+ * of nva_sample_static below) is counted in records of 2048 columns, the finest chunking any path
+ * has used; the present chunkings (4096 columns with a noise tensor, 8192 without) need fewer.
  */
 size_t nva_sample_workspace_bytes(int32_t batch, int32_t vocab);
 
@@ -217,6 +220,24 @@ int nva_rms_norm(const void *x, int64_t x_row_stride,
                  const void *residual, int64_t residual_row_stride,
                  const void *weight, void *out, void *residual_out,
                  int32_t rows, int32_t hidden, float eps, void *stream);
+
+/*
+ * Final norm of a prefill step on the rows that feed the LM head only.  Replaces the pair
+ * "hidden_states, _ = self.norm(hidden_states, residual)" (nanovllm/models/qwen3.py:176) +
+ * "x = x[cu_seqlens_q[1:] - 1].contiguous()" (nanovllm/layers/embed_head.py:56-61): the reference
+ * normalises all total_rows rows and then copies the last row of every sequence; this reads and
+ * normalises those batch rows alone, bit-identical to the rows nva_rms_norm would have produced.
+ *   i = cu_seqlens_q[b + 1] - 1  (a negative index wraps to total_rows + i, as torch indexing does;
+ *                                 an empty query span picks the previous sequence's last row, as in
+ *                                 the reference; indices are clamped to the tensor)
+ *   out[b] = bf16(s * rsqrt(mean(s^2) + eps)) * weight,  s = x[i] (+ residual[i] when residual != NULL)
+ * x / residual: bf16 [total_rows, hidden], row strides in elements; cu_seqlens_q: int32 [batch + 1];
+ * out: bf16 [batch, hidden] dense.  hidden % 8 == 0, hidden <= 4096.
+ */
+int nva_gather_last_rms_norm(const void *x, int64_t x_row_stride,
+                             const void *residual, int64_t residual_row_stride,
+                             const int32_t *cu_seqlens_q, const void *weight, void *out,
+                             int32_t batch, int32_t total_rows, int32_t hidden, float eps, void *stream);
 
 /*
  * Per-head RMSNorm of q and k followed by the neox rotary embedding, optionally fused with the

@@ -25,16 +25,25 @@ __device__ __forceinline__ float round_bf16(float v) { return bf16_to_f32(f32_to
 // use, so the kernel costs one memory round trip instead of one per chunk and tensor.
 // kResidual false: out = bf16(x * rsqrt(mean(x^2) + eps)) * w
 // else:            s = x + residual (fp32); residual_out = bf16(s); out = bf16(s * rsqrt(mean(s^2) + eps)) * w
-template <int NC, bool kResidual>
+// kGather: output row b is computed from input row ends[b + 1] - 1 (ends = the cumulative query
+// lengths of a prefill batch: the last token of sequence b), wrapped like a Python index when it is
+// negative; only those rows are read and no residual_out is written.
+template <int NC, bool kResidual, bool kGather>
 __global__ __launch_bounds__(256) void rms_norm_kernel(
     const bf16_t *__restrict__ x, int64_t x_stride, const bf16_t *__restrict__ residual, int64_t res_stride,
     const bf16_t *__restrict__ weight, bf16_t *__restrict__ out, bf16_t *__restrict__ residual_out,
-    int32_t rows, int32_t hidden, float eps) {
+    const int32_t *__restrict__ ends, int32_t src_rows, int32_t rows, int32_t hidden, float eps) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
-    const bf16_t *xr = x + static_cast<int64_t>(row) * x_stride;
-    const bf16_t *rr = kResidual ? residual + static_cast<int64_t>(row) * res_stride : nullptr;
+    int64_t src = row;
+    if (kGather) {
+        src = static_cast<int64_t>(ends[row + 1]) - 1;
+        if (src < 0) src += src_rows;                             // (x[-1] is the last row)
+        src = min(max(src, static_cast<int64_t>(0)), static_cast<int64_t>(src_rows) - 1);   // device data the host could not check
+    }
+    const bf16_t *xr = x + src * x_stride;
+    const bf16_t *rr = kResidual ? residual + src * res_stride : nullptr;
     uint4 xv[NC], rv[NC], wv[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
@@ -54,7 +63,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
             unpack8(rv[c], rf);
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[c][i] += rf[i];
-            if (live) {
+            if (live && !kGather) {
                 uint4 ro;
                 ro.x = pack_bf16x2(v[c][0], v[c][1]); ro.y = pack_bf16x2(v[c][2], v[c][3]);
                 ro.z = pack_bf16x2(v[c][4], v[c][5]); ro.w = pack_bf16x2(v[c][6], v[c][7]);
@@ -86,14 +95,35 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
 template <int NC>
 static void launch_rms_norm(hipStream_t stream, const bf16_t *x, int64_t x_stride, const bf16_t *residual,
                             int64_t res_stride, const bf16_t *weight, bf16_t *out, bf16_t *residual_out,
-                            int32_t rows, int32_t hidden, float eps) {
+                            const int32_t *ends, int32_t src_rows, int32_t rows, int32_t hidden, float eps) {
     const dim3 grid((rows + 3) / 4), block(256);
-    if (residual)
-        hipLaunchKernelGGL((rms_norm_kernel<NC, true>), grid, block, 0, stream, x, x_stride, residual, res_stride, weight,
-                           out, residual_out, rows, hidden, eps);
+    if (ends && residual)
+        hipLaunchKernelGGL((rms_norm_kernel<NC, true, true>), grid, block, 0, stream, x, x_stride, residual, res_stride,
+                           weight, out, residual_out, ends, src_rows, rows, hidden, eps);
+    else if (ends)
+        hipLaunchKernelGGL((rms_norm_kernel<NC, false, true>), grid, block, 0, stream, x, x_stride, residual, res_stride,
+                           weight, out, residual_out, ends, src_rows, rows, hidden, eps);
+    else if (residual)
+        hipLaunchKernelGGL((rms_norm_kernel<NC, true, false>), grid, block, 0, stream, x, x_stride, residual, res_stride,
+                           weight, out, residual_out, ends, src_rows, rows, hidden, eps);
     else
-        hipLaunchKernelGGL((rms_norm_kernel<NC, false>), grid, block, 0, stream, x, x_stride, residual, res_stride, weight,
-                           out, residual_out, rows, hidden, eps);
+        hipLaunchKernelGGL((rms_norm_kernel<NC, false, false>), grid, block, 0, stream, x, x_stride, residual, res_stride,
+                           weight, out, residual_out, ends, src_rows, rows, hidden, eps);
+}
+
+static void dispatch_rms_norm(hipStream_t st, const bf16_t *xp, int64_t x_row_stride, const bf16_t *rp,
+                              int64_t residual_row_stride, const bf16_t *wp, bf16_t *op, bf16_t *rop,
+                              const int32_t *ends, int32_t src_rows, int32_t rows, int32_t hidden, float eps) {
+    switch ((hidden + 511) / 512) {
+        case 1: launch_rms_norm<1>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, ends, src_rows, rows, hidden, eps); break;
+        case 2: launch_rms_norm<2>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, ends, src_rows, rows, hidden, eps); break;
+        case 3: launch_rms_norm<3>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, ends, src_rows, rows, hidden, eps); break;
+        case 4: launch_rms_norm<4>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, ends, src_rows, rows, hidden, eps); break;
+        case 5: launch_rms_norm<5>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, ends, src_rows, rows, hidden, eps); break;
+        case 6: launch_rms_norm<6>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, ends, src_rows, rows, hidden, eps); break;
+        case 7: launch_rms_norm<7>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, ends, src_rows, rows, hidden, eps); break;
+        default: launch_rms_norm<8>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, ends, src_rows, rows, hidden, eps); break;
+    }
 }
 
 // Eight lanes per (token, head) row of 128 elements: lane j of a row holds elements [8j, 8j+8) and
@@ -244,16 +274,27 @@ extern "C" int nva_rms_norm(const void *x, int64_t x_row_stride, const void *res
     const bf16_t *xp = static_cast<const bf16_t *>(x), *rp = static_cast<const bf16_t *>(residual);
     const bf16_t *wp = static_cast<const bf16_t *>(weight);
     bf16_t *op = static_cast<bf16_t *>(out), *rop = static_cast<bf16_t *>(residual_out);
-    switch ((hidden + 511) / 512) {
-        case 1: launch_rms_norm<1>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
-        case 2: launch_rms_norm<2>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
-        case 3: launch_rms_norm<3>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
-        case 4: launch_rms_norm<4>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
-        case 5: launch_rms_norm<5>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
-        case 6: launch_rms_norm<6>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
-        case 7: launch_rms_norm<7>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
-        default: launch_rms_norm<8>(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, rows, hidden, eps); break;
-    }
+    dispatch_rms_norm(st, xp, x_row_stride, rp, residual_row_stride, wp, op, rop, nullptr, rows, rows, hidden, eps);
+    return launch_status();
+}
+
+extern "C" int nva_gather_last_rms_norm(const void *x, int64_t x_row_stride, const void *residual,
+                                        int64_t residual_row_stride, const int32_t *cu_seqlens_q, const void *weight,
+                                        void *out, int32_t batch, int32_t total_rows, int32_t hidden, float eps,
+                                        void *stream) {
+    using namespace nva;
+    if (batch < 0 || total_rows < 0 || hidden <= 0) return NVA_ERR_BAD_SHAPE;
+    if (hidden % 8 != 0 || hidden > kNormMaxChunks * 512) return NVA_ERR_UNSUPPORTED_GEOMETRY;
+    if (batch == 0) return NVA_OK;
+    if (total_rows == 0) return NVA_ERR_BAD_SHAPE;                 // rows to pick, none to pick from
+    if (!x || !weight || !out || !cu_seqlens_q) return NVA_ERR_NULL_POINTER;
+    if (x_row_stride < hidden || x_row_stride % 8 != 0) return NVA_ERR_BAD_STRIDE;
+    if (residual && (residual_row_stride < hidden || residual_row_stride % 8 != 0)) return NVA_ERR_BAD_STRIDE;
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(out) || (residual && !aligned16(residual)))
+        return NVA_ERR_MISALIGNED;
+    dispatch_rms_norm(static_cast<hipStream_t>(stream), static_cast<const bf16_t *>(x), x_row_stride,
+                      static_cast<const bf16_t *>(residual), residual_row_stride, static_cast<const bf16_t *>(weight),
+                      static_cast<bf16_t *>(out), nullptr, cu_seqlens_q, total_rows, batch, hidden, eps);
     return launch_status();
 }
 

@@ -41,6 +41,7 @@ SIGNATURES = {
                                           _f32, _vp]),
     "nva_sample_workspace_bytes": (_sz, [_i32, _i32]),
     "nva_rms_norm": (C.c_int, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _f32, _vp]),
+    "nva_gather_last_rms_norm": (C.c_int, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _vp]),
     "nva_qk_norm_rope": (C.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i64,
                                    _i32, _i32, _i32, _i32, _f32, _vp]),
     "nva_silu_and_mul": (C.c_int, [_vp, _i64, _vp, _i32, _i32, _vp]),

@@ -40,6 +40,25 @@ def add_rms_norm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, 
     return out, res_out
 
 
+def gather_last_rms_norm(x: torch.Tensor, residual, cu_seqlens_q: torch.Tensor, weight: torch.Tensor,
+                         eps: float) -> torch.Tensor:
+    """Final (add +) RMSNorm of the last row of every sequence of a prefill batch: the rows
+    ``x[cu_seqlens_q[1:] - 1]`` of nanovllm/layers/embed_head.py:58-60, normalised as
+    nanovllm/models/qwen3.py:176 does for all rows -- without touching the others."""
+    assert x.dim() == 2 and x.dtype == _BF16 and x.stride(1) == 1 and x.is_cuda
+    assert cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.is_contiguous() and cu_seqlens_q.is_cuda
+    batch = cu_seqlens_q.numel() - 1
+    out = torch.empty((max(batch, 0), x.shape[1]), dtype=_BF16, device=x.device)
+    if residual is not None:
+        assert residual.shape == x.shape and residual.dtype == _BF16 and residual.stride(1) == 1
+    rc = _lib.load().nva_gather_last_rms_norm(
+        x.data_ptr(), x.stride(0), None if residual is None else residual.data_ptr(),
+        0 if residual is None else residual.stride(0), cu_seqlens_q.data_ptr(), weight.data_ptr(),
+        out.data_ptr(), batch, x.shape[0], x.shape[1], float(eps), _stream())
+    _lib.check(rc, "nva_gather_last_rms_norm")
+    return out
+
+
 def build_rope_cache(head_dim: int, max_position: int, base: float, device) -> torch.Tensor:
     """``[max_position, head_dim]`` fp32: cos in the first half of a row, sin in the second
     (the table of nanovllm/layers/rotary_embedding.py:28-35)."""

@@ -88,6 +88,15 @@ class Qwen3ForCausalLM(nn.Module):
         hidden, _ = layers.add_rms_norm(hidden, residual, self.norm, self.cfg.rms_norm_eps)
         return hidden
 
+    def prefill_logits(self, input_ids: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        """``compute_logits(forward(...))`` of a prefill step with the final norm applied to the
+        rows the LM head reads only: the last token of every sequence
+        (nanovllm/models/qwen3.py:176, nanovllm/layers/embed_head.py:56-61)."""
+        hidden, residual = self.forward_layers(input_ids, positions, None, None, 0, len(self.layers))
+        rows = layers.gather_last_rms_norm(hidden, residual, get_context().cu_seqlens_q, self.norm,
+                                           self.cfg.rms_norm_eps)
+        return F.linear(rows, self.lm_head)
+
     def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
         """Logits of the last token of every sequence (nanovllm/layers/embed_head.py:56-61)."""
         ctx = get_context()

@@ -302,6 +302,8 @@ class ModelRunner:
 
     @torch.inference_mode()
     def run_model(self, input_ids: torch.Tensor, positions: torch.Tensor, is_prefill: bool) -> torch.Tensor:
+        if is_prefill:                                            # final norm on the last row of every sequence only
+            return self.model.prefill_logits(input_ids, positions)
         return self.model.compute_logits(self.model(input_ids, positions))
 
     def run(self, seqs: List[Sequence], is_prefill: bool) -> List[int]:

@@ -6,6 +6,8 @@ Each function follows the reference line by line, including where it rounds to b
   apply_rope, qk_norm_rope  nanovllm/layers/rotary_embedding.py:6-15,37-48 and
                             nanovllm/models/qwen3.py:74-79
   silu_and_mul              nanovllm/layers/activation.py:11-14
+  last_token_norm           nanovllm/models/qwen3.py:176 (final norm over all rows) followed by
+                            nanovllm/layers/embed_head.py:58-60 (rows cu_seqlens_q[1:] - 1)
   build_rope_cache          nanovllm/layers/rotary_embedding.py:28-35 (cos | sin table)
 """
 import torch
@@ -27,6 +29,14 @@ def add_rms_norm(x, residual, weight, eps):
     var = xf.pow(2).mean(dim=-1, keepdim=True)
     xf = xf * torch.rsqrt(var + eps)
     return xf.to(orig) * weight, new_residual
+
+
+def last_token_norm(x, residual, cu_seqlens_q, weight, eps):
+    """What the LM head receives in a prefill step: the final norm of every row, then the last
+    row of every sequence (torch indexing: a negative index counts from the end)."""
+    normed = rms_norm(x, weight, eps) if residual is None else add_rms_norm(x, residual, weight, eps)[0]
+    last_indices = cu_seqlens_q[1:].long() - 1
+    return normed[last_indices].contiguous()
 
 
 def build_rope_cache(head_dim, max_position, base):

@@ -141,6 +141,21 @@ def test_sampler_validation_and_workspace_size():
     assert f(A, 100, A, None, 0, 0, 0, A, A, 1 << 20, 0, 100, None) == _lib.OK
 
 
+def test_gather_last_rms_norm_validation():
+    f = _lib.load().nva_gather_last_rms_norm
+    assert f(None, 1024, A, 1024, A, A, A, 4, 100, 1024, 1e-6, None) == _lib.ERR_NULL_POINTER
+    assert f(A, 1024, A, 1024, None, A, A, 4, 100, 1024, 1e-6, None) == _lib.ERR_NULL_POINTER    # cu_seqlens_q
+    assert f(A, 1024, A, 1024, A, A, None, 4, 100, 1024, 1e-6, None) == _lib.ERR_NULL_POINTER    # out
+    assert f(A, 1024, A, 1024, A, A, A, -1, 100, 1024, 1e-6, None) == _lib.ERR_BAD_SHAPE
+    assert f(A, 1024, A, 1024, A, A, A, 4, 0, 1024, 1e-6, None) == _lib.ERR_BAD_SHAPE            # rows to pick from nothing
+    assert f(A, 1000, A, 1024, A, A, A, 4, 100, 1024, 1e-6, None) == _lib.ERR_BAD_STRIDE
+    assert f(A, 1024, A, 1028, A, A, A, 4, 100, 1024, 1e-6, None) == _lib.ERR_BAD_STRIDE
+    assert f(A + 4, 1024, A, 1024, A, A, A, 4, 100, 1024, 1e-6, None) == _lib.ERR_MISALIGNED
+    assert f(A, 1024, A, 1024, A, A, A, 4, 100, 1020, 1e-6, None) == _lib.ERR_UNSUPPORTED_GEOMETRY
+    assert f(A, 8192, A, 8192, A, A, A, 4, 100, 8192, 1e-6, None) == _lib.ERR_UNSUPPORTED_GEOMETRY
+    assert f(None, 0, None, 0, None, None, None, 0, 0, 1024, 1e-6, None) == _lib.OK               # empty batch
+
+
 def test_stage_decode_inputs_validation():
     f = _lib.load().nva_stage_decode_inputs
     # (dst, src_host, nbytes, ids_offset, index_offset, n, prev_tokens, n_prev, stream)

@@ -40,6 +40,45 @@ def test_rms_norm_and_add_rms_norm(dev, rows, hidden):
     assert_bf16_close(out2, want, "add_rms_norm")
 
 
+@pytest.mark.parametrize("batch,total,hidden", [(29, 16384, 1024), (4, 700, 4096), (1, 1, 1024), (7, 50, 1000)])
+def test_gather_last_rms_norm_is_the_full_norm_at_the_last_rows(dev, batch, total, hidden):
+    """The final norm on the last token of every sequence only (what the LM head of a prefill step
+    reads) against the oracle's full norm followed by the gather, with and without a residual; and
+    bit for bit the rows the full-size kernel produces."""
+    g = torch.Generator().manual_seed(batch * 31 + hidden)
+    x = (torch.randn(total, hidden, generator=g) * 3).to(torch.bfloat16)
+    r = torch.randn(total, hidden, generator=g).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(torch.bfloat16)
+    cuts = torch.sort(torch.randperm(total - 1, generator=g)[: batch - 1] + 1).values if batch > 1 else torch.empty(0, dtype=torch.long)
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), cuts, torch.tensor([total])]).to(torch.int32)
+    got = layers.gather_last_rms_norm(x.to(dev), r.to(dev), cu.to(dev), w.to(dev), 1e-6)
+    assert got.shape == (batch, hidden)
+    assert_bf16_close(got, glue.last_token_norm(x, r, cu, w, 1e-6), "gather + add + norm")
+    full, _ = layers.add_rms_norm(x.to(dev), r.to(dev), w.to(dev), 1e-6)
+    assert torch.equal(got, full[(cu[1:] - 1).long().to(dev)])
+    got = layers.gather_last_rms_norm(x.to(dev), None, cu.to(dev), w.to(dev), 1e-6)
+    assert_bf16_close(got, glue.last_token_norm(x, None, cu, w, 1e-6), "gather + norm")
+
+
+def test_gather_last_rms_norm_empty_spans_and_strided_rows(dev):
+    """An empty query span picks the previous sequence's last row and an empty FIRST span wraps to
+    the last row of the tensor, as the reference's ``x[cu_seqlens_q[1:] - 1]`` does; rows may be
+    strided views; a bound beyond the tensor is clamped instead of read out of bounds."""
+    g = torch.Generator().manual_seed(5)
+    wide = torch.randn(40, 2048, generator=g).to(torch.bfloat16)
+    r = torch.randn(40, 1024, generator=g).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(1024, generator=g)).to(torch.bfloat16)
+    x = wide[:, 512:1536]
+    cu = torch.tensor([0, 0, 13, 13, 40], dtype=torch.int32)
+    got = layers.gather_last_rms_norm(wide.to(dev)[:, 512:1536], r.to(dev), cu.to(dev), w.to(dev), 1e-6)
+    assert_bf16_close(got, glue.last_token_norm(x, r, cu, w, 1e-6), "empty spans")
+    assert torch.equal(got[1], got[2]) and not torch.equal(got[0], got[1])
+    beyond = torch.tensor([0, 13, 900], dtype=torch.int32)
+    got = layers.gather_last_rms_norm(wide.to(dev)[:, 512:1536], r.to(dev), beyond.to(dev), w.to(dev), 1e-6)
+    want = glue.last_token_norm(x, r, torch.tensor([0, 13, 40], dtype=torch.int32), w, 1e-6)
+    assert_bf16_close(got, want, "clamped bound")
+
+
 def test_rms_norm_strided_rows(dev):
     g = torch.Generator().manual_seed(9)
     wide = torch.randn(16, 2048, generator=g).to(torch.bfloat16)

@@ -36,6 +36,25 @@ def test_add_rms_norm_is_norm_of_the_sum_and_returns_rounded_sum():
     assert torch.equal(glue.add_rms_norm(x, torch.zeros_like(x), w, 1e-6)[0], glue.rms_norm(x, w, 1e-6))
 
 
+def test_last_token_norm_rows_by_float64_loop():
+    """Row b of the result is the norm of input row cu[b+1]-1, computed here element by element in
+    float64 without the restatement's code; an empty span repeats the previous row, index -1 wraps."""
+    g = torch.Generator().manual_seed(4)
+    x, r = torch.randn(9, 64, generator=g).to(torch.bfloat16), torch.randn(9, 64, generator=g).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(64, generator=g)).to(torch.bfloat16)
+    cu = torch.tensor([0, 0, 3, 3, 8, 9], dtype=torch.int32)          # spans: empty (wraps to row 8), 3, empty, 5, 1
+    out = glue.last_token_norm(x, r, cu, w, 1e-6)
+    assert out.shape == (5, 64)
+    for b, src in enumerate([8, 2, 2, 7, 8]):
+        s = [float(x[src, i]) + float(r[src, i]) for i in range(64)]
+        inv = 1.0 / math.sqrt(sum(v * v for v in s) / 64 + 1e-6)
+        for i in range(64):
+            want = s[i] * inv * float(w[i])
+            assert abs(float(out[b, i]) - want) <= 2.0 ** -6 * max(abs(want), 1e-3), (b, i)
+    # without a residual the plain norm of the same rows
+    assert torch.equal(glue.last_token_norm(x, None, cu, w, 1e-6), glue.rms_norm(x, w, 1e-6)[[8, 2, 2, 7, 8]])
+
+
 def test_rope_table_and_rotation_properties():
     cache = glue.build_rope_cache(128, 64, 1e6)
     assert cache.shape == (64, 128)
