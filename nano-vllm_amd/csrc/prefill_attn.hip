@@ -445,9 +445,14 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_kernel(const Prefi
             if (kPaged && !tile_ok) step(kt, yes, no, yes);     // (a tile behind a bad block id is masked out: nothing to add)
             else step(kt, no, yes, yes);
         }
-        for (; kt < min(n_active, last); ++kt) step(kt, yes, yes, yes);
+        for (; kt < min(n_active, last); ++kt) {
+            // (behind a bad block id the loads were pointed at block 0, which may never have been written:
+            // with every score masked the products would still be 0 x its contents, and 0 x NaN is NaN)
+            if (kPaged && !tile_ok) step(kt, yes, no, yes);
+            else step(kt, yes, yes, yes);
+        }
         for (; kt < last; ++kt) step(kt, yes, no, yes);
-        if (last >= 0 && last < n_active) step(last, yes, yes, no);    // (with the mask, needed or not: one body fewer)
+        if (last >= 0 && last < n_active && !(kPaged && !tile_ok)) step(last, yes, yes, no);    // (with the mask, needed or not: one body fewer)
         if (kExact) {
 #pragma unroll
             for (int qa = 0; qa < 2; ++qa) {

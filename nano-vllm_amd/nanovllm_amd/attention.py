@@ -62,6 +62,7 @@ def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor,
 
 _workspaces: dict = {}
 _retired_workspaces: list = []
+_last_builder: dict = {}                 # device -> the DecodePlan (or None) of the last call that derived a work split there
 
 
 def _decode_workspace(device, nbytes: int) -> torch.Tensor:
@@ -126,8 +127,12 @@ def paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
             plan.key = key
         elif plan.key != key:
             raise ValueError("decode plan reused with a different batch, geometry, table or workspace")
-        else:
+        elif _last_builder.get(q.device) is plan:
             mode = _PLAN_REUSE
+        # else: another decode call derived its own split in the shared workspace since this plan's
+        # first call and overwrote the stored one -- derive it again
+    if mode == _PLAN_BUILD:
+        _last_builder[q.device] = plan
     rc = lib.nva_paged_decode_attn_planned(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                            block_tables.data_ptr(), block_tables.stride(0), max_blocks,
                                            context_lens.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),

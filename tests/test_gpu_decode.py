@@ -185,6 +185,26 @@ def test_decode_plan_reuse_is_bit_identical(dev, shape):
         assert torch.equal(paged_decode_attention(*od, other.scale, plan=plan), o_alone)
 
 
+def test_decode_plan_survives_another_batch_in_between(dev):
+    """All decode calls of a device share one workspace, the stored work split included.  A call on
+    another batch between a plan's first call and a later one overwrites the split; the later call
+    must notice and derive its own again instead of following the other batch's records."""
+    a = synthetic.decode_case(seed=90, batch=24, num_blocks=128, ctx_lo=1, ctx_hi=1200)
+    b = synthetic.decode_case(seed=91, batch=9, num_blocks=128, ctx_lo=300, ctx_hi=3000)
+    da = (a.q.to(dev), a.k_cache.to(dev), a.v_cache.to(dev), a.context_lens.to(dev), a.block_tables.to(dev))
+    db = (b.q.to(dev), b.k_cache.to(dev), b.v_cache.to(dev), b.context_lens.to(dev), b.block_tables.to(dev))
+    want_a = paged_decode_attention(*da, a.scale).clone()
+    want_b = paged_decode_attention(*db, b.scale).clone()
+    assert_attn_close(want_a, _oracle(a), "batch a")
+    plan_a, plan_b = DecodePlan(), DecodePlan()
+    assert torch.equal(paged_decode_attention(*da, a.scale, plan=plan_a), want_a)      # builds
+    assert torch.equal(paged_decode_attention(*db, b.scale, plan=plan_b), want_b)      # builds over it
+    assert torch.equal(paged_decode_attention(*da, a.scale, plan=plan_a), want_a)      # must rebuild
+    assert torch.equal(paged_decode_attention(*da, a.scale, plan=plan_a), want_a)      # reuses its own again
+    assert torch.equal(paged_decode_attention(*db, b.scale), want_b)                   # a call without a plan builds too
+    assert torch.equal(paged_decode_attention(*da, a.scale, plan=plan_a), want_a)
+
+
 def test_decode_batch_above_one_launch(dev):
     """More than 1024 sequences run as two launches sharing the workspace; a stored work split is
     then never reused (each launch overwrites it), with or without a plan object."""

@@ -235,3 +235,42 @@ def test_lookahead_decode_produces_the_same_tokens(dev):
             assert ids[-1] == eos or len(ids) == p.max_tokens
         assert any(ids[-1] == eos and len(ids) < p.max_tokens for ids, p in zip(run, params))
     assert [r[:1] for r in stopped[True]] == [r[:1] for r in runs[True]]
+
+
+def test_bench_request_mix_at_full_request_count(dev):
+    """The 256 requests of the end-to-end benchmark (prompt lengths U[100,1024] over the whole
+    vocabulary, temperature 0.6, ignore_eos) on the full Qwen3-0.6B architecture with hipGraph
+    decode, output lengths divided by 8 to keep the run short: every request returns exactly
+    ``max_tokens`` ids inside the vocabulary, every KV block is back on the free list afterwards,
+    the bucket accounting adds up, and a second generate() on newly drawn ids of the same lengths
+    gives the same counts."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    from nanovllm_amd.engine import qwen3_0_6b
+    prompts, params = bench.e2e_workload()
+    assert len(prompts) == 256 and min(map(len, prompts)) >= 100 and max(map(len, prompts)) <= 1024
+    for p in params:
+        p.max_tokens = max(1, p.max_tokens // 8)
+    llm = LLM(qwen3_0_6b(), enforce_eager=False, max_model_len=4096, num_kvcache_blocks=2048)
+    mr, bm = llm.model_runner, llm.scheduler.block_manager
+    assert mr.graph_bs[-1] == 512 and 256 in mr.graph_bs
+    for round_ in range(2):
+        used0, replayed0 = mr.bucket_rows
+        steps0 = llm.stats["decode_steps"]
+        outs = llm.generate(bench.fresh_prompts(prompts, 100 + round_), params)
+        assert len(outs) == 256
+        for o, p in zip(outs, params):
+            assert len(o["token_ids"]) == p.max_tokens
+            assert all(0 <= t < 151936 for t in o["token_ids"])
+        assert len(bm.free_block_ids) == 2048 and not bm.used_block_ids       # every block was released
+        assert not llm.scheduler.running and not llm.scheduler.waiting
+        used, replayed = mr.bucket_rows[0] - used0, mr.bucket_rows[1] - replayed0
+        # every sampled token but the one the prefill step produces comes from one decode row
+        # (a launched-ahead step may add rows for sequences that had just finished: none here, ignore_eos)
+        assert used == sum(p.max_tokens - 1 for p in params), (used, sum(p.max_tokens - 1 for p in params))
+        assert used <= replayed <= used + 15 * (llm.stats["decode_steps"] - steps0)      # padding below one bucket step per step
+        assert llm.stats["decode_steps"] - steps0 >= max(p.max_tokens for p in params) - 1
+    # different prompts, same temperature: the sampled tokens differ between the rounds
+    assert outs[0]["token_ids"] != [0] * len(outs[0]["token_ids"])

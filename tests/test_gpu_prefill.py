@@ -141,6 +141,46 @@ def test_prefill_bad_table_entry_contributes_nothing(dev):
     assert_attn_close(out, want, "bad table entries")
 
 
+@pytest.mark.parametrize("bad_col", [0, 1])
+def test_prefill_bad_table_entry_on_a_diagonal_tile_over_an_unwritten_cache(dev, bad_col):
+    """A bad block id behind NEW tokens: its key tiles cross the causal diagonal (and one is the last
+    tile of its query tile).  Every row of the caches that no token was written to -- block 0 above
+    all, where a bad id's loads are pointed -- holds NaN bit patterns, as an engine's torch.empty
+    cache may; the block's keys must drop out without a single NaN reaching the output."""
+    g = torch.Generator().manual_seed(31 + bad_col)
+    lq, hq, hkv, d = 300, 16, 8, 128
+    q, k, v = (torch.randn(lq, h, d, generator=g).to(torch.bfloat16) for h in (hq, hkv, hkv))
+    blocks = [3, 5]
+    pos = torch.arange(lq)
+    slots = (torch.tensor(blocks)[pos // 256] * 256 + pos % 256).to(torch.int32)
+    kc = torch.full((8, 256, hkv, d), float("nan"), dtype=torch.bfloat16, device=dev)
+    vc = torch.full_like(kc, float("nan"))
+    store_kvcache(k.to(dev), v.to(dev), kc, vc, slots.to(dev))
+    table = torch.tensor([blocks], dtype=torch.int32)
+    table[0, bad_col] = 9999 if bad_col else -1
+    cu = torch.tensor([0, lq], dtype=torch.int32)
+    out = varlen_prefill_attention(q.to(dev), kc, vc, cu.to(dev), cu.to(dev), lq, lq, d ** -0.5, block_table=table.to(dev))
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out.float()).all()), "NaN from an unwritten block reached the output"
+    scale = d ** -0.5
+    if bad_col == 1:
+        # keys 256.. drop out: queries below 256 are untouched, the others see keys 0..255, all of them
+        cu256 = torch.tensor([0, 256], dtype=torch.int32)
+        low = oracle.varlen_prefill_attention(q[:256], k[:256], v[:256], cu256, cu256, scale, precision="fp32")
+        n = lq - 256
+        cu_q1 = torch.arange(n + 1, dtype=torch.int32)
+        cu_k1 = (torch.arange(n + 1) * 256).to(torch.int32)
+        high = oracle.varlen_prefill_attention(q[256:], k[:256].repeat(n, 1, 1), v[:256].repeat(n, 1, 1), cu_q1, cu_k1,
+                                               scale, precision="fp32")
+        want = torch.cat([low, high])
+    else:
+        # keys 0..255 drop out: queries below 256 see nothing (zero rows), the others the keys from 256 on, causally
+        cu_t = torch.tensor([0, lq - 256], dtype=torch.int32)
+        high = oracle.varlen_prefill_attention(q[256:], k[256:], v[256:], cu_t, cu_t, scale, precision="fp32")
+        want = torch.cat([torch.zeros(256, hq, d), high])
+    assert_attn_close(out, want, f"bad id in column {bad_col}")
+
+
 def test_prefill_sequences_do_not_leak(dev):
     case = synthetic.prefill_case(seed=6, batch=3, prefix_fraction=0.0, q_lo=50, q_hi=200)
     out, _ = _packed(case, dev)

@@ -49,6 +49,55 @@ def test_sample_static_matches_sample_on_two_calls_in_a_row(dev, with_noise):
     assert torch.equal(big, again) and small.numel() == 7
 
 
+def test_sample_static_takes_no_device_memory_and_replays_from_a_graph(dev):
+    """After a first call has looked the scratch array up: (1) the free device memory the driver
+    reports is the same before and after a call -- the caching allocator's own counter would not see
+    a hipMalloc inside the library; (2) the call can be captured in a HIP graph, and every replay, on
+    new logits and with eager work and synchronisation in between, gives what nva_sample gives."""
+    lib = _lib.load()
+    batch, vocab, seed, offset = 64, 151936, 5, 9
+    g = torch.Generator().manual_seed(123)
+    logits = (torch.randn(batch, vocab, generator=g) * 2).to(torch.bfloat16).to(dev)
+    temps = torch.full((batch,), 0.8, device=dev)
+    out = torch.full((batch,), -1, dtype=torch.int64, device=dev)
+    want = torch.full((batch,), -2, dtype=torch.int64, device=dev)
+    ws = torch.empty(lib.nva_sample_workspace_bytes(batch, vocab), dtype=torch.uint8, device=dev)
+
+    def static_call():
+        rc = lib.nva_sample_static(logits.data_ptr(), logits.stride(0), temps.data_ptr(), None, 0, seed, offset,
+                                   out.data_ptr(), batch, vocab, torch.cuda.current_stream().cuda_stream)
+        assert rc == _lib.OK, _lib.status_string(rc)
+
+    def eager_reference():
+        rc = lib.nva_sample(logits.data_ptr(), logits.stride(0), temps.data_ptr(), None, 0, seed, offset,
+                            want.data_ptr(), ws.data_ptr(), ws.numel(), batch, vocab,
+                            torch.cuda.current_stream().cuda_stream)
+        assert rc == _lib.OK, _lib.status_string(rc)
+
+    static_call()                                                        # warm: address look-up, code object load
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    static_call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_call()
+    seen = set()
+    for replay in range(4):
+        logits.copy_((torch.randn(batch, vocab, generator=g) * 2).to(torch.bfloat16))
+        out.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager_reference()                                                # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), replay
+        assert int(out.min()) >= 0 and int(out.max()) < vocab
+        seen.add(tuple(out[:8].tolist()))
+    assert len(seen) == 4                                                # the replays really saw different logits
+
+
 def test_sample_static_rejects_what_does_not_fit(dev):
     """Inputs and outputs are real tensors: a library that wrongly accepted the call would still touch only memory it may."""
     lib = _lib.load()
