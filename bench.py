@@ -522,6 +522,19 @@ def stream_read_us(dev, nbytes, steps=60, graph=False):
     return ms / steps * 1e3
 
 
+def device_copy_us(dev, nbytes, steps=400):
+    """Microseconds the runtime's own device-to-device copy of `nbytes` takes (reads nbytes, writes nbytes), as one
+    replayed hipGraph of the copies, rotating through buffers that together exceed the Infinity Cache: the attainable
+    side of the kernels that read and write in equal parts (the scatters)."""
+    import torch
+    nbytes = nbytes // 16 * 16
+    n_buf = max(2, -(-(400 << 20) // nbytes))
+    src = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(n_buf)]
+    dst = [torch.empty_like(b) for b in src]
+    ms, _ = _graph_time_ms([lambda a=a, b=b: b.copy_(a) for a, b in zip(src, dst)], steps, 5)
+    return ms / steps * 1e3
+
+
 def bench_read_probe(args, dev):
     """What a bare streaming read costs at the sizes of the bandwidth-bound kernels' workloads."""
     sizes = {"scatter_config1 (read half of 31.9 MB)": 15_945_728, "sampler 256 x 151,936": 77_791_232,
@@ -590,7 +603,11 @@ def collect_extra(dev, model, prompts, params):
     extra["attainable"] = {"what": "us per launch of a bare streaming read of the same bytes (nva_probe_stream_read)",
                            "decode_config2_291MB_us": round(stream_read_us(dev, extra["decode_config2"]["algorithmic_bytes_per_launch"]), 2),
                            "sampler_78MB_us": round(stream_read_us(dev, extra["sampler_256x151936"]["algorithmic_bytes_per_launch"]), 2),
-                           "decode_config5_shape_us": round(stream_read_us(dev, extra["decode_config5_shape"]["algorithmic_bytes_per_launch"], steps=12), 2)}
+                           "decode_config5_shape_us": round(stream_read_us(dev, extra["decode_config5_shape"]["algorithmic_bytes_per_launch"], steps=12), 2),
+                           "decode_e2e_shape_855MB_us": round(stream_read_us(dev, 855_318_528, steps=40), 2),
+                           "scatter_config1_read_16MB_us": round(stream_read_us(dev, extra["scatter_config1"]["algorithmic_bytes_per_launch"] // 2, steps=400, graph=True), 2),
+                           "scatter_config1_copy_16MB_to_16MB_us": round(device_copy_us(dev, extra["scatter_config1"]["algorithmic_bytes_per_launch"] // 2), 2),
+                           "rope_scatter_copy_155MB_to_155MB_us": round(device_copy_us(dev, extra["rope_scatter_16384_tokens"]["algorithmic_bytes_per_launch"] // 2, steps=100), 2)}
     gc.collect()
     torch.cuda.empty_cache()
     llm = LLM(model, enforce_eager=True, max_model_len=4096, num_kvcache_blocks=4096)
@@ -601,6 +618,18 @@ def collect_extra(dev, model, prompts, params):
                           "what": "the same 256-request workload with enforce_eager=True (no hipGraph decode), one pass",
                           "prefill_s": round(llm.stats["prefill_s"], 3), "decode_s": round(llm.stats["decode_s"], 3)}
     del llm
+    gc.collect()
+    torch.cuda.empty_cache()
+    # config 5 end to end (Qwen3-8B architecture, batch 128, contexts U[4096,16384], 128 decode steps, greedy + T=1.0):
+    # one warm-up pass and one timed pass of the engine, no profiler attached
+    t0 = time.perf_counter()
+    res, _ = bench_longctx(SimpleNamespace(steps=1, warmup=1, eager=False, requests=128), dev)
+    extra["longctx_e2e"] = {"value": res["value"], "unit": "tok/s", "ms_per_decode_step": res["config"]["ms_per_decode_step"],
+                            "kv_gbps_over_the_whole_step": res["roofline"]["achieved"], "frac_of_hbm_peak": res["roofline"]["frac"],
+                            "kv_bytes_per_decode_step": res["config"]["kv_bytes_per_decode_step"],
+                            "kv_cache_bytes": res["config"]["kv_cache_bytes"], "kv_cache_blocks": res["config"]["kv_cache_blocks"],
+                            "what": res["config"]["workload"] + "; one timed pass of 128 engine decode steps after one warm-up pass",
+                            "wall_s_including_setup": round(time.perf_counter() - t0, 1)}
     gc.collect()
     torch.cuda.empty_cache()
     return extra
@@ -620,16 +649,32 @@ def bench_e2e(args, dev):
     llm.generate([[1, 2, 3, 4]], SamplingParams(max_tokens=8, ignore_eos=True))     # reference warm-up call
     for w in range(args.warmup):
         llm.generate(fresh_prompts(prompts[:32], 9_000 + w), params[:32])
+    mr = llm.model_runner
+    mr.decode_step_events, kv_tokens0 = [], mr.kv_tokens_attended          # per-step HIP events from here on
     dt = _e2e_passes(llm, prompts, params, args.steps, 0)
     tok_s = total_out * args.steps / dt
+    # what the decode steps of the timed passes really read: every step attends over sum(context_lens) tokens in
+    # every layer (K and V rows of all kv heads); their GPU time is taken from a pair of events around every step
+    decode_gpu_s = sum(a.elapsed_time(b) for a, b in mr.decode_step_events) * 1e-3
+    n_decode_steps = len(mr.decode_step_events)
+    mr.decode_step_events = None
+    kv_bytes = (mr.kv_tokens_attended - kv_tokens0) * model.num_hidden_layers * model.num_key_value_heads * model.head_dim * 2 * 2
 
     layers = [m for m in llm.model_runner.model.modules() if isinstance(m, nva.Attention)]
     roof = decode_e2e_shape_roofline(dev, [(a.k_cache, a.v_cache) for a in layers], llm.config.num_kvcache_blocks)
+    in_run_gbps = kv_bytes / decode_gpu_s / 1e9
+    roof["in_run"] = {"what": "K/V bytes the decode steps of the timed passes attended over (sum of context_lens x layers x kv heads "
+                              "x 128 x 2 B x 2) / GPU time of those steps (HIP events around every step: staging, 28 layers with "
+                              "GEMMs, norms and attention, LM head, sampler) -- the whole step, not the attention kernel alone",
+                      "kv_bytes_per_pass": kv_bytes // args.steps, "decode_steps_per_pass": n_decode_steps // args.steps,
+                      "decode_gpu_s_per_pass": round(decode_gpu_s / args.steps, 4),
+                      "mean_kv_bytes_per_attention_launch": kv_bytes // max(n_decode_steps * model.num_hidden_layers, 1),
+                      "achieved": round(in_run_gbps, 1), "unit": "GB/s", "frac": round(in_run_gbps / HBM_PEAK_GBPS, 4)}
     st = dict(llm.stats)
     used, replayed = llm.model_runner.bucket_rows
     buckets = {"graph_bucket_step": llm.config.graph_bucket_step, "decode_rows_used": used, "decode_rows_replayed": replayed,
                "padded_fraction": round(1 - used / max(replayed, 1), 4)}
-    del layers, llm
+    del layers, llm, mr
     gc.collect()
     torch.cuda.empty_cache()
     result = {
@@ -641,7 +686,7 @@ def bench_e2e(args, dev):
                                + ("eager" if args.eager else "hipGraph decode"),
                    "requests": args.requests, "output_tokens": total_out, "engine_steps_per_pass": (st["prefill_steps"] + st["decode_steps"]) // args.steps,
                    "prefill_s_per_pass": round(st["prefill_s"] / args.steps, 3), "decode_s_per_pass": round(st["decode_s"] / args.steps, 3),
-                   "decode_buckets": buckets},
+                   "decode_buckets": buckets, "kv_bytes_per_pass": kv_bytes // args.steps},
         "roofline": roof,
     }
     if not args.no_extra:
@@ -675,8 +720,9 @@ def bench_longctx(args, dev):
     n_req, n_steps = args.requests if args.requests != 256 else 128, 128
     ctx = [rng.randint(4096, 16384) for _ in range(n_req)]
     need = sum(-(-(c + n_steps) // 256) for c in ctx)
+    # (every request runs the same 128 steps, so only the full batch size is ever replayed: no intermediate graph buckets)
     llm = LLM(model, enforce_eager=args.eager, max_model_len=16384 + 256, max_num_batched_tokens=32768,
-              max_num_seqs=n_req, num_kvcache_blocks=need + 8)
+              max_num_seqs=n_req, num_kvcache_blocks=need + 8, graph_bucket_step=max(n_req, 1))
     mr, sch = llm.model_runner, llm.scheduler
     with torch.inference_mode():
         for l in range(model.num_hidden_layers):                 # synthetic KV content
@@ -732,7 +778,8 @@ def bench_longctx(args, dev):
                                "%d randomly scattered 256-token blocks (%.1f GB cache), 128 decode steps, greedy + T=1.0, %s"
                                % (n_req, sum(ctx) // n_req, need, (need + 8) * 37.75e6 / 1e9,
                                   "eager" if args.eager else "hipGraph decode"),
-                   "ms_per_decode_step": round(dt / n_steps * 1e3, 2)},
+                   "ms_per_decode_step": round(dt / n_steps * 1e3, 2), "kv_cache_blocks": need + 8,
+                   "kv_cache_bytes": int(mr.kv_cache.numel()) * 2, "kv_bytes_per_decode_step": kv_bytes_per_step},
         "roofline": {"bound": "hbm", "achieved": round(kv_bytes_per_step / (dt / n_steps) / 1e9, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(kv_bytes_per_step / (dt / n_steps) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
                      "kernel": "whole decode step (36 x decode_stream_kernel<4> dominate): KV bytes of one step / step time",

@@ -22,6 +22,9 @@ from .model import Qwen3ForCausalLM
 from .sequence import PENDING_TOKEN, Sequence
 
 
+_capture_anchor: list = []       # see ModelRunner.__init__
+
+
 @dataclass
 class DecodeHandle:
     """A decode step that has been enqueued but whose tokens have not been read back."""
@@ -109,8 +112,20 @@ class ModelRunner:
         self.graphs = {}
         self.graph_bs: List[int] = []
         self.bucket_rows = [0, 0]                        # decode rows used / rows replayed (bucket padding), since start
+        self.kv_tokens_attended = 0                      # sum of context lengths over all decode steps, since start
+        self.decode_step_events = None                   # a list: (start, end) HIP events of every decode step are appended
         self.graph_segments = 4                          # consecutive graphs per decode step (see capture_graphs)
         self._graph_keepalive = []
+        if not self.enforce_eager and not torch.is_inference_mode_enabled() and not _capture_anchor:
+            # torch allocates the default generator's graph bookkeeping tensors when the first live graph
+            # registers and updates them in place at every later capture: allocated under inference mode
+            # (where the decode graphs are captured) they would make every capture outside it fail for
+            # as long as those graphs live.  One small graph captured here and kept for the life of the
+            # process pins them as ordinary tensors.
+            probe, one = torch.cuda.CUDAGraph(), torch.ones(1, device=self.device)
+            with torch.cuda.graph(probe):
+                one = one + 1
+            _capture_anchor.append((probe, one))
         with torch.inference_mode():
             self.warmup_model()
             self.allocate_kv_cache()
@@ -251,6 +266,7 @@ class ModelRunner:
         self.bucket_rows[0] += bs                                 # rows that carry a sequence / rows replayed
         self.bucket_rows[1] += bucket
         h = build_decode_inputs(seqs, self.block_size)
+        self.kv_tokens_attended += int(h["context_lens"].sum(dtype=np.int64))
         self._stage_turn ^= 1
         st = self._stage_np[self._stage_turn]
         pending = h["input_ids"] == PENDING_TOKEN
@@ -291,8 +307,10 @@ class ModelRunner:
         """Enqueue one decode step and its sampling; nothing is read back.  ``prev`` is the step
         launched before, if its tokens have not been committed to the sequences yet."""
         with torch.inference_mode():
+            started = self._step_started()
             logits = self._run_decode_graph(seqs, prev)
             tokens_dev = self.sampler(logits, self.graph_vars["temperatures"][: len(seqs)])
+            self._step_ended(started)
             tokens_host = self._tokens_host[self._stage_turn]
             tokens_host[: len(seqs)].copy_(tokens_dev, non_blocking=True)
             ready = torch.cuda.Event()
@@ -306,8 +324,23 @@ class ModelRunner:
             return self.model.prefill_logits(input_ids, positions)
         return self.model.compute_logits(self.model(input_ids, positions))
 
+    def _step_started(self):
+        """Start event of a decode step when the caller asked for step timings (``decode_step_events``)."""
+        if self.decode_step_events is None:
+            return None
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        return ev
+
+    def _step_ended(self, started) -> None:
+        if started is not None:
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            self.decode_step_events.append((started, ev))
+
     def run(self, seqs: List[Sequence], is_prefill: bool) -> List[int]:
         with torch.inference_mode():
+            started = None if is_prefill else self._step_started()
             if not is_prefill and self.graph_bs and len(seqs) <= self.graph_bs[-1]:
                 logits = self._run_decode_graph(seqs)
                 temperatures = self.graph_vars["temperatures"][: len(seqs)]
@@ -316,10 +349,13 @@ class ModelRunner:
                     input_ids, positions = self.prepare_prefill(seqs)
                     temperatures = self._pf_temperatures          # staged with the other prefill inputs
                 else:
+                    self.kv_tokens_attended += sum(len(s) for s in seqs)
                     input_ids, positions = self.prepare_decode(seqs)
                     temperatures = self.prepare_sample(seqs)
                 logits = self.run_model(input_ids, positions, is_prefill)
-            tokens = self.sampler(logits, temperatures).tolist()   # the one device->host sync per step
+            tokens_dev = self.sampler(logits, temperatures)
+            self._step_ended(started)
+            tokens = tokens_dev.tolist()                           # the one device->host sync per step
         reset_context()
         return tokens
 
