@@ -262,13 +262,18 @@ def bench_sampler(args, dev):
         sets.append(logits)
     temps = torch.full((batch,), 0.6, device=dev)
     with_noise = bool(getattr(args, "noise", False))
+    # the engine's sampler call: records in the library's built-in scratch (nva_sample_static, no allocation);
+    # `--workspace`: nva_sample with a workspace tensor allocated per call
+    static = not bool(getattr(args, "workspace", False))
     if with_noise:                                   # the replayable path: an Exp(1) tensor per set of logits is read as well
         noises = [torch.empty((batch, vocab), device=dev).exponential_(1.0, generator=g) for _ in sets]
-        fns = [lambda l=l, n=n: nva.sample(l, temps, n) for l, n in zip(sets, noises)]
+        mk = lambda st: [lambda l=l, n=n: nva.sample(l, temps, n, static_scratch=st) for l, n in zip(sets, noises)]
     else:
-        fns = [lambda l=l, i=i: nva.sample(l, temps, None, seed=1, offset=i) for i, l in enumerate(sets)]
-    ms = _event_time_ms(fns, args.steps, args.warmup)
+        mk = lambda st: [lambda l=l, i=i: nva.sample(l, temps, None, seed=1, offset=i, static_scratch=st) for i, l in enumerate(sets)]
+    ms = _event_time_ms(mk(static), args.steps, args.warmup)
     per_step_ms = ms / args.steps
+    other_us = _event_time_ms(mk(not static), args.steps, args.warmup) / args.steps * 1e3
+
     alg = batch * vocab * (6 if with_noise else 2)
     gbps = alg / (per_step_ms * 1e-3) / 1e9
     result = {
@@ -282,7 +287,8 @@ def bench_sampler(args, dev):
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
                      "kernel": ("sampler_chunk_kernel<2, true>" if with_noise else "sampler_chunk_kernel<4, false>") + " + sampler_row_kernel",
-                     "algorithmic_bytes_per_launch": alg},
+                     "algorithmic_bytes_per_launch": alg,
+                     ("us_per_launch_with_workspace_tensor" if static else "us_per_launch_static_scratch"): round(other_us, 2)},
     }
 
     def cpu():
@@ -803,6 +809,7 @@ def main():
     ap.add_argument("--requests", type=int, default=256, help="e2e only: number of requests (profiling runs)")
     ap.add_argument("--max-output-len", type=int, default=1024, help="e2e only: cap on output lengths (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workspace", action="store_true", help="sampler: the two-kernel form with a workspace tensor (nva_sample) instead of nva_sample_static")
     ap.add_argument("--tokens", type=int, default=None, help="scatter / rope-scatter: number of tokens (default 4096 / 16384)")
     ap.add_argument("--contiguous", action="store_true", help="scatter: slots in ascending order instead of a random permutation")
     ap.add_argument("--noise", action="store_true", help="sampler: time the replayable path that reads an Exp(1) noise tensor")

@@ -3,11 +3,28 @@ import pytest
 import torch
 
 import oracle
-from nanovllm_amd import sample, Sampler
+from nanovllm_amd import Sampler
+from nanovllm_amd import sample as _sample
 from nanovllm_amd import synthetic
 from helpers import assert_sampled_like_oracle
 
 pytestmark = pytest.mark.gpu
+
+_mode = {"static": False}
+
+
+def sample(*args, **kw):
+    kw.setdefault("static_scratch", _mode["static"])
+    return _sample(*args, **kw)
+
+
+@pytest.fixture(autouse=True, params=[False, True], ids=["workspace", "static"])
+def _scratch_mode(request):
+    """Every test runs twice: through nva_sample (workspace tensor) and through nva_sample_static
+    (records in the library's own array, what the engine's Sampler module calls)."""
+    _mode["static"] = request.param
+    yield
+    _mode["static"] = False
 
 
 def _check(case, dev):
