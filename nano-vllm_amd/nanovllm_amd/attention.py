@@ -184,6 +184,20 @@ def varlen_prefill_attention(q: torch.Tensor, k: Optional[torch.Tensor], v: Opti
     return out
 
 
+def _decode_plan_of(ctx) -> Optional[DecodePlan]:
+    """The work-split plan the layers of this forward pass share: the one on the context, made here by
+    the first layer if the runner did not provide any.  Eager runs and graph captures never share one."""
+    capturing = torch.cuda.is_current_stream_capturing()
+    plan = getattr(ctx, "decode_plan", None)
+    if plan is None or plan.capturing != capturing:
+        plan = DecodePlan(capturing)
+        try:
+            ctx.decode_plan = plan
+        except AttributeError:                     # a foreign context object without room for it: no sharing
+            return None
+    return plan
+
+
 class Attention(nn.Module):
     """Paged-KV attention layer: scatter the new K/V rows, then prefill or decode attention.
 
@@ -215,4 +229,4 @@ class Attention(nn.Module):
                 ctx.cu_seqlens_q, ctx.cu_seqlens_k, ctx.max_seqlen_q, ctx.max_seqlen_k,
                 self.scale, block_table=ctx.block_tables)
         return paged_decode_attention(q, k_cache, v_cache, ctx.context_lens, ctx.block_tables, self.scale,
-                                      plan=getattr(ctx, "decode_plan", None))
+                                      plan=_decode_plan_of(ctx))

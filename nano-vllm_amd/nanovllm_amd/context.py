@@ -17,16 +17,21 @@ import torch
 class DecodePlan:
     """Marks the decode-attention calls that share one work split: the layers of one decode
     step, which see the same ``context_lens`` and ``block_tables``.  The first call made with
-    a plan derives the split, the later ones take it from the workspace.  A runner opts in by
-    putting a fresh plan on the context for every forward pass (and for every graph capture,
-    after the eager warm-up); without one every call derives its own split, which is what a
-    runner that reuses one ``Context`` for warm-up and capture (nanovllm/engine/model_runner.py:
-    229-237) needs.
-    """
-    __slots__ = ("key",)
+    a plan derives the split, the later ones take it from the workspace.
 
-    def __init__(self):
+    A runner may put a fresh plan on the context for every forward pass itself.  If it does not,
+    the attention layer keeps one on the ``Context`` object it is handed: all layers of a forward
+    pass see the same object, and the runner installs a new one for every step (``set_context``
+    replaces the context wholesale, nanovllm/utils/context.py:21-23).  A plan made outside graph
+    capture is never used inside one and vice versa (``capturing``): the reference warms a batch
+    size up and captures it under one ``Context`` (nanovllm/engine/model_runner.py:229-237), and a
+    captured layer must not rely on a split that only the warm-up run derived.
+    """
+    __slots__ = ("key", "capturing")
+
+    def __init__(self, capturing: bool = False):
         self.key = None        # (workspace address, batch, heads, kv heads) of the call that built it
+        self.capturing = capturing
 
 
 @dataclass

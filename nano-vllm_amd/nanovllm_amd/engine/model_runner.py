@@ -385,7 +385,7 @@ class ModelRunner:
             outputs[:bs] = self.model(input_ids[:bs], positions[:bs])        # eager warm-up (sizes workspaces)
             # the captured layers share one work split of the decode kernel: the first layer derives
             # it at every replay, the others take it from the workspace
-            get_context().decode_plan = DecodePlan()
+            get_context().decode_plan = DecodePlan(capturing=True)
             segments, hidden, residual = [], None, None
             for first, last in zip(cuts[:-1], cuts[1:]):
                 graph = torch.cuda.CUDAGraph()

@@ -106,3 +106,62 @@ def test_graph_replays_match_eager_calls_and_the_oracle(dev, shared_split):
         assert not got[0][live:].any() and not got[1][live:].any(), "rows without keys must be zero"
         greedy = new["logits"].float().argmax(-1)
         assert torch.equal(got[4].cpu()[::6], greedy[::6])
+
+
+def test_attention_module_under_the_reference_capture_pattern(dev):
+    """nanovllm/engine/model_runner.py:229-237 installs ONE context per batch size, runs the model once
+    eagerly (warm-up) and once more under graph capture, then replays the graph on new contents of the
+    same tensors.  Three Attention layers driven that way, with no plan supplied by the runner: the
+    layers share a work split on their own (the first derives it, the others reuse it), the captured
+    layers must not lean on the split the warm-up run left behind, and every replay must equal the
+    eager result of a fresh context and stay within tolerance of the oracle."""
+    import nanovllm_amd as nva
+    from nanovllm_amd.context import get_context
+    g = torch.Generator().manual_seed(5)
+    n_layers = 3
+    pools = [(torch.randn(BLOCKS, 256, HKV, D, generator=g).to(torch.bfloat16).to(dev),
+              torch.randn(BLOCKS, 256, HKV, D, generator=g).to(torch.bfloat16).to(dev)) for _ in range(n_layers)]
+    attn = []
+    for kc, vc in pools:
+        layer = nva.Attention(HQ, D, D ** -0.5, HKV)
+        layer.k_cache, layer.v_cache = kc, vc
+        attn.append(layer)
+    st = {k: v.to(dev) for k, v in _draw(300, dev, B).items()}
+    qs = [torch.randn(B, HQ, D, generator=g).to(torch.bfloat16).to(dev) for _ in range(n_layers)]
+
+    def forward():
+        return [layer(q, st["k"], st["v"]).clone() for layer, q in zip(attn, qs)]
+
+    nva.set_context(False, slot_mapping=st["slots"], context_lens=st["ctx"], block_tables=st["tables"])
+    forward()                                                          # warm-up under the context ...
+    warm_plan = get_context().decode_plan
+    assert warm_plan is not None and not warm_plan.capturing           # ... whose layers shared a split
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):                                      # ... and capture under the same one
+        captured = forward()
+    assert get_context().decode_plan is not warm_plan and get_context().decode_plan.capturing
+    nva.reset_context()
+    torch.cuda.synchronize()
+    for r, live in enumerate([B, 5, 17]):
+        new = _draw(400 + r, dev, live)
+        for name, value in new.items():
+            st[name].copy_(value.to(dev))
+        before = [(kc.clone(), vc.clone()) for kc, vc in pools]
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        for (kc, vc), (bk, bv) in zip(pools, before):
+            kc.copy_(bk)
+            vc.copy_(bv)
+        nva.set_context(False, slot_mapping=st["slots"], context_lens=st["ctx"], block_tables=st["tables"])
+        want = forward()                                               # a fresh context: builds, then reuses
+        nva.reset_context()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), f"replay {r}: layer {i} differs from the eager call"
+        ek, ev = before[0][0].cpu(), before[0][1].cpu()
+        oracle.store_kvcache(new["k"], new["v"], ek, ev, new["slots"])
+        ref = oracle.paged_decode_attention(qs[0][:live].cpu(), ek, ev, new["ctx"][:live], new["tables"][:live], D ** -0.5, "fp32")
+        assert_attn_close(got[0][:live, 0], ref, f"replay {r} layer 0")
