@@ -340,7 +340,22 @@ def bench_glue(args, dev):
             r = torch.randn(n, hidden, device=dev, generator=g).to(torch.bfloat16)
             fns.append(lambda x=x, r=r: layers.add_rms_norm(x, r, w, 1e-6))
         alg = n * hidden * 2 * 4 + hidden * 2            # x and the residual in, both results out
-        kernel = "rms_norm_kernel<2, true>"
+        kernel = "rms_norm_kernel<2, true, false>"
+    elif which == "last-token-norm":
+        # the final norm of a prefill step: 29 sequences in a batch of n rows; only their last rows feed the LM head
+        w = torch.ones(hidden, dtype=torch.bfloat16, device=dev)
+        batch = 29
+        cu = torch.linspace(0, n, batch + 1).to(torch.int32).to(dev)
+        full = bool(getattr(args, "grid_order", False))   # (--grid-order here: the reference's order -- norm every row, then gather)
+        for _ in range(3):
+            x = torch.randn(n, hidden, device=dev, generator=g).to(torch.bfloat16)
+            r = torch.randn(n, hidden, device=dev, generator=g).to(torch.bfloat16)
+            if full:
+                fns.append(lambda x=x, r=r: layers.add_rms_norm(x, r, w, 1e-6)[0][(cu[1:] - 1).long()].contiguous())
+            else:
+                fns.append(lambda x=x, r=r: layers.gather_last_rms_norm(x, r, cu, w, 1e-6))
+        alg = batch * hidden * 2 * 3 + hidden * 2 + (batch + 1) * 4     # the picked rows of x and the residual in, their norm out
+        kernel = "rms_norm_kernel<2, true, false> over all rows + index kernels" if full else "rms_norm_kernel<2, true, true>"
     else:
         for _ in range(3):
             x = torch.randn(n, 2 * inter, device=dev, generator=g).to(torch.bfloat16)
@@ -830,11 +845,12 @@ def main():
     ap.add_argument("--requests", type=int, default=256, help="e2e only: number of requests (profiling runs)")
     ap.add_argument("--max-output-len", type=int, default=1024, help="e2e only: cap on output lengths (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--grid-order", action="store_true", help="glue last-token-norm: norm every row, then gather (the reference's order) instead of the gathering kernel")
     ap.add_argument("--workspace", action="store_true", help="sampler: the two-kernel form with a workspace tensor (nva_sample) instead of nva_sample_static")
     ap.add_argument("--tokens", type=int, default=None, help="scatter / rope-scatter: number of tokens (default 4096 / 16384)")
     ap.add_argument("--contiguous", action="store_true", help="scatter: slots in ascending order instead of a random permutation")
     ap.add_argument("--noise", action="store_true", help="sampler: time the replayable path that reads an Exp(1) noise tensor")
-    ap.add_argument("--glue", choices=["add-rms-norm", "silu-mul"], default="add-rms-norm", help="glue: which elementwise kernel")
+    ap.add_argument("--glue", choices=["add-rms-norm", "silu-mul", "last-token-norm"], default="add-rms-norm", help="glue: which elementwise kernel")
     ap.add_argument("--uniform", default=None, metavar="SxL", help="prefill: S packed sequences of L tokens each instead of config 3 (e.g. 2x16384)")
     ap.add_argument("--bucket-step", type=int, default=16, help="e2e only: spacing of the captured decode batch sizes")
     ap.add_argument("--no-extra", action="store_true", help="e2e only: skip the per-configuration rooflines and the eager pass")
